@@ -1,0 +1,195 @@
+"""The cache manager: page pools per group of layers, block tables per request,
+slots for fixed-size per-request state, and the device storage behind them.
+
+Needs come from the model (``CausalLM.cache_needs()``), one per schedule entry.
+Entries with equal KV needs (kv heads, head size, window) form a group with a
+page pool of its own; every group has its own block tables, so a windowed group
+can give pages back while a full group keeps them.  Entries with equal state
+needs form a state group.  Device layout of a KV group:
+``k, v : [entries, pages, kv_heads, page_size, head_dim]`` in the model's dtype; a
+token's slot number is ``page * page_size + position % page_size``
+(qil/cache.py:79-82).  Storage is never cleared: kernels read only positions below a
+request's computed length and inside its window (qil/cache.py:127-128,137;
+tests fill the pool with NaN).
+
+Per request the manager keeps ``computed``: how many tokens every layer has
+cached.  A step must start exactly there (qil/cache.py:84-95,113-116) and
+``advance`` moves it after the step ran.
+"""
+from collections import deque
+from dataclasses import dataclass
+
+import torch
+
+from ..parts.base import KVNeed, StateNeed
+from .pages import PagePool, CacheFull
+
+
+@dataclass
+class KVView:
+    """What an attention-like mixer sees of its schedule entry's cache in one step."""
+    k: torch.Tensor              # [pages, kv_heads, page_size, head_dim]
+    v: torch.Tensor
+    page_size: int
+    writes: bool                 # False for an entry that reads another entry's cache
+    group: int
+    block_tables: torch.Tensor = None    # int32 [n_seqs, stride], filled per step
+    slots: torch.Tensor = None           # int32 [n_tokens], slot of each new token
+
+
+@dataclass
+class StateView:
+    """Fixed-size state of a schedule entry: ``state[slot]`` belongs to one live request."""
+    state: torch.Tensor          # [slots, *shape]
+    writes: bool
+    group: int
+
+
+class CacheManager:
+    def __init__(self, needs, *, num_pages, page_size, max_requests, dtype=torch.float32, device='cpu',
+                 max_step_tokens=None, allocate=True):
+        self.page_size, self.max_requests, self.dtype, self.device = page_size, max_requests, dtype, torch.device(device)
+        self.kv_groups, self.state_groups = [], []     # dicts: need, entries, pool / need, entries
+        self.binding = []                              # per schedule entry: None | (kind, group, index, writes)
+        for position, need in enumerate(needs):
+            if need is None:
+                self.binding.append(None)
+            elif isinstance(need, tuple) and need[0] == 'shared':
+                kind, group, index, _ = self.binding[need[1]]
+                self.binding.append((kind, group, index, False))
+            elif isinstance(need, KVNeed):
+                group = self._group(self.kv_groups, need)
+                self.binding.append(('kv', group, len(self.kv_groups[group]['entries']), True))
+                self.kv_groups[group]['entries'].append(position)
+            elif isinstance(need, StateNeed):
+                group = self._group(self.state_groups, need)
+                self.binding.append(('state', group, len(self.state_groups[group]['entries']), True))
+                self.state_groups[group]['entries'].append(position)
+            else:
+                raise TypeError(f'unknown cache need {need!r}')
+        pages = num_pages if isinstance(num_pages, (list, tuple)) else [num_pages] * len(self.kv_groups)
+        if len(pages) != len(self.kv_groups):
+            raise ValueError(f'{len(self.kv_groups)} page groups, {len(pages)} page counts')
+        for group, count in zip(self.kv_groups, pages):
+            group['pool'] = PagePool(num_pages=count, page_size=page_size, window=group['need'].window,
+                                     max_step_tokens=max_step_tokens)
+        self.free_slots = deque(range(max_requests))
+        self.slots, self.computed, self.limits = {}, {}, {}
+        if allocate:
+            self._allocate()
+
+    @staticmethod
+    def _group(groups, need):
+        for index, group in enumerate(groups):
+            if group['need'] == need:
+                return index
+        groups.append(dict(need=need, entries=[]))
+        return len(groups) - 1
+
+    def _allocate(self):
+        for group in self.kv_groups:
+            need, pool = group['need'], group['pool']
+            shape = (len(group['entries']), pool.capacity, need.kv_heads, self.page_size, need.head_dim)
+            group['k'] = torch.empty(shape, dtype=self.dtype, device=self.device)
+            group['v'] = torch.empty(shape, dtype=self.dtype, device=self.device)
+        for group in self.state_groups:
+            need = group['need']
+            dtype = torch.float32 if need.dtype == 'float32' else self.dtype
+            group['state'] = torch.zeros((len(group['entries']), self.max_requests, *need.shape),
+                                         dtype=dtype, device=self.device)
+
+    # ------------------------------------------------------------------ requests
+    def pages_for(self, tokens):
+        return (tokens + self.page_size - 1) // self.page_size
+
+    def fits_at_all(self, tokens):
+        """Could a request of ``tokens`` cached tokens ever be admitted (empty cache)?"""
+        return all(g['pool'].reservation_for(tokens) <= g['pool'].capacity for g in self.kv_groups)
+
+    def admit(self, request, max_cached_tokens=None):
+        """Reserve credits in every group and a state slot; False if they do not fit now.
+
+        ``max_cached_tokens`` None admits without reservation (trace replay, where a
+        request's length is not known ahead): ``ensure`` may then raise CacheFull.
+        """
+        if request in self.slots:
+            raise ValueError('duplicate cache owner')
+        if max_cached_tokens is not None and (type(max_cached_tokens) is not int or max_cached_tokens < 1):
+            raise ValueError('cache reservation must be a positive integer')
+        if not self.free_slots or not all(g['pool'].can_admit(max_cached_tokens) for g in self.kv_groups):
+            return False
+        for group in self.kv_groups:
+            group['pool'].admit(request, max_cached_tokens)
+        self.slots[request] = self.free_slots.popleft()
+        self.computed[request] = 0
+        self.limits[request] = max_cached_tokens
+        return True
+
+    def ensure(self, request, end):
+        """Physical pages for positions below ``end`` in every group (all or nothing)."""
+        limit = self.limits[request]
+        if end <= 0 or (limit is not None and end > limit):
+            raise ValueError('write exceeds reserved context')
+        short = [g for g in self.kv_groups
+                 if g['pool'].pages_for(end) - len(g['pool'].tables[request]) > len(g['pool'].free)]
+        if short:
+            if limit is not None:
+                raise RuntimeError('cache reservation invariant violated')    # qil/cache.py:75-76
+            raise CacheFull(f'out of pages for request {request!r} at {end} tokens')
+        for group in self.kv_groups:
+            group['pool'].ensure(request, end)
+
+    def advance(self, request, end):
+        """The step has cached tokens up to ``end``; windows give passed pages back."""
+        if end < self.computed[request]:
+            raise ValueError('computed length cannot shrink')
+        self.computed[request] = end
+        for group in self.kv_groups:
+            group['pool'].pass_window(request, end)
+
+    def release(self, request):
+        if request not in self.slots:
+            raise ValueError('unknown cache owner')
+        for group in self.kv_groups:
+            group['pool'].release(request)
+        self.free_slots.append(self.slots.pop(request))
+        del self.computed[request], self.limits[request]
+
+    def owns(self, request):
+        return request in self.slots
+
+    def table(self, group, request):
+        return self.kv_groups[group]['pool'].tables[request]
+
+    @property
+    def free_pages(self):
+        return [len(g['pool'].free) for g in self.kv_groups]
+
+    def check(self):
+        for group in self.kv_groups:
+            group['pool'].check()
+            if set(group['pool'].tables) != set(self.slots):
+                raise AssertionError('pools and slots disagree about live requests')
+        slots = sorted(list(self.free_slots) + list(self.slots.values()))
+        if slots != list(range(self.max_requests)):
+            raise AssertionError(f'state slots broken: {slots}')
+
+    # ------------------------------------------------------------------ views
+    def views(self):
+        """One view per schedule entry (None where the mixer keeps nothing)."""
+        out = []
+        for bound in self.binding:
+            if bound is None:
+                out.append(None)
+                continue
+            kind, group, index, writes = bound
+            if kind == 'kv':
+                g = self.kv_groups[group]
+                out.append(KVView(g['k'][index], g['v'][index], self.page_size, writes, group))
+            else:
+                out.append(StateView(self.state_groups[group]['state'][index], writes, group))
+        return out
+
+    def bytes_per_token(self):
+        size = torch.empty((), dtype=self.dtype).element_size()
+        return sum(2 * len(g['entries']) * g['need'].kv_heads * g['need'].head_dim * size for g in self.kv_groups)

@@ -1,0 +1,252 @@
+// Split-context attention of single query rows over the paged cache, and the merge of the splits.
+//
+// Every token of the step is a row with its own visible range of keys:
+//   [lo, ctx) with ctx = position + 1, lo = window > 0 ? max(0, ctx - window) : 0
+// (key j visible iff j <= position, qil/model.py:62-64).  A decoded token is one row; the tokens of a
+// prompt portion are rows sharing a block table, whose keys were written before this kernel runs.
+//
+// Partial kernel: grid (rows, kv_heads, parts), 256 threads.  A block owns the keys
+// [part * P, (part + 1) * P) of one row and one kv head and serves the whole group of query heads
+// that read this kv head (h // g, qil/model.py:59-61), so K and V are read once per group rather
+// than once per query head (the reference's kernel reads them per query head:
+// qil/paged_attention.py:13-41).  Scores, maxima, exponentials, sums and weighted values are
+// float32 (qil/paged_attention.py:27-41).  A block whose range is empty returns without writing,
+// and the merge skips the same parts (qil/paged_attention.py:33-34 handles it with a safe maximum).
+// With a single part the normalised result is written directly.
+//
+// Merge kernel: grid (rows, heads): out = sum_p acc_p exp(m_p - m) / sum_p l_p exp(m_p - m)
+// (qil/paged_attention.py:44-58).
+//
+// Lanes: a token's d elements are spread over TG = next_pow2(ceil(d / 8)) lanes, eight elements a
+// lane; a wave handles 64 / TG tokens at a time.
+#include "common.h"
+
+#define ATT_THREADS 256
+#define ATT_WAVES (ATT_THREADS / QIL_WAVE)
+
+template <typename T, int GT>
+__global__ void __launch_bounds__(ATT_THREADS)
+attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
+                         const T* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
+                         const int* __restrict__ row_seq, const int* __restrict__ positions,
+                         float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l,
+                         T* __restrict__ out, int heads, int kv_heads, int d, int page_size, int window,
+                         float scale, int P, int parts, int tg_log2) {
+  extern __shared__ float lds[];
+  const int row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
+  const int g = heads / kv_heads;
+  const int ctx = positions[row] + 1;
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int begin = max(part * P, lo), end = min((part + 1) * P, ctx);
+  if (begin >= end) return;
+  const int count = end - begin;
+
+  const int TG = 1 << tg_log2, TPW = QIL_WAVE >> tg_log2;
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int sub = lane & (TG - 1), slot = lane >> tg_log2;
+  const int e0 = sub * 8;
+  const bool live = e0 < d;                       // lanes past d (padding of TG to a power of two) idle
+  const int* table = block_tables + (size_t)row_seq[row] * table_stride;
+
+  float* scores = lds;                            // [GT][P]
+  float* reduce = lds + GT * P;                   // [16] block reductions
+  float* wave_acc = reduce + 16;                  // [ATT_WAVES][GT][d]
+
+  for (int h0 = 0; h0 < g; h0 += GT) {
+    // ---- scores of this head tile against the block's keys
+    float qv[GT][8];
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      const int head = kvh * g + h0 + h;
+      if (live && h0 + h < g) ld8(q + (size_t)row * q_stride + (size_t)head * d + e0, qv[h]);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[h][e] = 0.f;
+    }
+    for (int t = wave * TPW + slot; t < count; t += ATT_WAVES * TPW) {
+      const int j = begin + t;
+      const size_t page = table[j / page_size];
+      const size_t base = ((page * kv_heads + kvh) * page_size + (j % page_size)) * (size_t)d + e0;
+      float kv[8];
+      if (live) ld8(k_cache + base, kv);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; ++e) kv[e] = 0.f;
+#pragma unroll
+      for (int h = 0; h < GT; ++h) {
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot += qv[h][e] * kv[e];
+        for (int o = TG >> 1; o > 0; o >>= 1) dot += __shfl_xor(dot, o, QIL_WAVE);
+        if (sub == 0) scores[h * P + t] = dot * scale;
+      }
+    }
+    __syncthreads();
+
+    // ---- softmax statistics per head (block wide), probabilities back into LDS
+    float m_h[GT], l_h[GT];
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      float m = -INFINITY;
+      for (int t = threadIdx.x; t < count; t += ATT_THREADS) m = fmaxf(m, scores[h * P + t]);
+      m = block_max(m, reduce);
+      float l = 0.f;
+      for (int t = threadIdx.x; t < count; t += ATT_THREADS) {
+        const float p = expf(scores[h * P + t] - m);
+        scores[h * P + t] = p;
+        l += p;
+      }
+      l = block_sum(l, reduce);
+      m_h[h] = m;
+      l_h[h] = l;
+    }
+    __syncthreads();
+
+    // ---- weighted values
+    float acc[GT][8];
+#pragma unroll
+    for (int h = 0; h < GT; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
+    for (int t = wave * TPW + slot; t < count; t += ATT_WAVES * TPW) {
+      const int j = begin + t;
+      const size_t page = table[j / page_size];
+      const size_t base = ((page * kv_heads + kvh) * page_size + (j % page_size)) * (size_t)d + e0;
+      float vv[8];
+      if (live) ld8(v_cache + base, vv);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vv[e] = 0.f;
+#pragma unroll
+      for (int h = 0; h < GT; ++h) {
+        const float p = scores[h * P + t];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] += p * vv[e];
+      }
+    }
+    // sum over the token slots of the wave, then over the waves (fixed order)
+#pragma unroll
+    for (int h = 0; h < GT; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        for (int o = TG; o < QIL_WAVE; o <<= 1) acc[h][e] += __shfl_xor(acc[h][e], o, QIL_WAVE);
+    if (slot == 0 && live) {
+#pragma unroll
+      for (int h = 0; h < GT; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wave_acc[(wave * GT + h) * d + e0 + e] = acc[h][e];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < GT * d; idx += ATT_THREADS) {
+      const int h = idx / d, e = idx - h * d;
+      if (h0 + h >= g) continue;
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < ATT_WAVES; ++w) total += wave_acc[(w * GT + h) * d + e];
+      const int head = kvh * g + h0 + h;
+      // m_h / l_h live in registers indexed by a compile-time h; select without dynamic indexing
+      float m = 0.f, l = 1.f;
+#pragma unroll
+      for (int hh = 0; hh < GT; ++hh)
+        if (hh == h) { m = m_h[hh]; l = l_h[hh]; }
+      if (parts == 1) {
+        st(out + ((size_t)row * heads + head) * d + e, total / l);
+      } else {
+        const size_t cell = ((size_t)row * heads + head) * parts + part;
+        part_acc[cell * d + e] = total;
+        if (e == 0) { part_m[cell] = m; part_l[cell] = l; }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+__global__ void attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
+                                       const float* __restrict__ part_l, const int* __restrict__ positions,
+                                       T* __restrict__ out, int heads, int d, int window, int P, int parts) {
+  const int row = blockIdx.x, head = blockIdx.y;
+  const int ctx = positions[row] + 1;
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int first = lo / P, last = (ctx - 1) / P;
+  const size_t cell0 = ((size_t)row * heads + head) * parts;
+  float m = -INFINITY;
+  for (int p = first; p <= last; ++p) m = fmaxf(m, part_m[cell0 + p]);
+  float denom = 0.f;
+  for (int p = first; p <= last; ++p) denom += part_l[cell0 + p] * expf(part_m[cell0 + p] - m);
+  for (int e = threadIdx.x; e < d; e += blockDim.x) {
+    float numer = 0.f;
+    for (int p = first; p <= last; ++p) numer += part_acc[(cell0 + p) * d + e] * expf(part_m[cell0 + p] - m);
+    st(out + ((size_t)row * heads + head) * d + e, numer / denom);
+  }
+}
+
+static int next_pow2_log2(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return l;
+}
+
+// LDS floats the partial kernel needs.
+static size_t rows_lds_floats(int gt, int P, int d) { return (size_t)gt * P + 16 + (size_t)ATT_WAVES * gt * d; }
+
+template <typename T>
+static int launch_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                       int table_stride, const int* row_seq, const int* positions, float* part_acc, float* part_m,
+                       float* part_l, void* out, int rows, int heads, int kv_heads, int d, int page_size, int window,
+                       float scale, int P, int parts, hipStream_t s) {
+  const int g = heads / kv_heads;
+  const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;            // head tile: 1, 2, 4 or 8
+  const int tg_log2 = next_pow2_log2((d + 7) / 8);
+  const size_t lds = rows_lds_floats(gt, P, d) * sizeof(float);
+  dim3 grid(rows, kv_heads, parts);
+#define QIL_ROWS_CASE(GT)                                                                                          \
+  hipLaunchKernelGGL((attn_rows_partial_kernel<T, GT>), grid, dim3(ATT_THREADS), lds, s, (const T*)q, q_stride,    \
+                     (const T*)k_cache, (const T*)v_cache, block_tables, table_stride, row_seq, positions,         \
+                     part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, P, parts,    \
+                     tg_log2)
+  switch (gt) {
+    case 1: QIL_ROWS_CASE(1); break;
+    case 2: QIL_ROWS_CASE(2); break;
+    case 4: QIL_ROWS_CASE(4); break;
+    default: QIL_ROWS_CASE(8); break;
+  }
+#undef QIL_ROWS_CASE
+  int status = (int)hipGetLastError();
+  if (status || parts == 1) return status;
+  hipLaunchKernelGGL(attn_rows_merge_kernel<T>, dim3(rows, heads), dim3(d >= 128 ? 128 : 64), 0, s, part_acc, part_m,
+                     part_l, positions, (T*)out, heads, d, window, P, parts);
+  return (int)hipGetLastError();
+}
+
+extern "C" {
+
+// Bytes of float32 workspace for `rows` rows split into `parts` parts (0 when parts == 1).
+size_t qil_attn_rows_workspace(int rows, int heads, int d, int parts) {
+  return parts <= 1 ? 0 : (size_t)rows * heads * parts * (d + 2) * sizeof(float);
+}
+
+// q: rows of stride q_stride elements, head h at offset h * d.  out: [rows, heads * d].
+// workspace: qil_attn_rows_workspace bytes.  P: keys per part, parts = ceil(max context / P).
+// Requires d % 8 == 0, d <= 256, P <= 1024.  Returns -1 on a size it does not take.
+int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                  int table_stride, const int* row_seq, const int* positions, void* workspace, void* out, int rows,
+                  int heads, int kv_heads, int d, int page_size, int window, float scale, int P, int parts, int dtype,
+                  hipStream_t s) {
+  if (rows == 0) return 0;
+  if (d % 8 || d > 256 || d < 8 || heads % kv_heads || P < 1 || P > 1024 || parts < 1 || parts > 65535 ||
+      kv_heads > 65535) return -1;
+  const int g = heads / kv_heads;
+  const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;
+  if (rows_lds_floats(gt, P, d) * sizeof(float) > 64 * 1024) return -1;
+  float* acc = (float*)workspace;
+  float* m = acc ? acc + (size_t)rows * heads * parts * d : nullptr;
+  float* l = m ? m + (size_t)rows * heads * parts : nullptr;
+  if (dtype == QIL_F32)
+    return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, acc, m, l,
+                              out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+  return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, acc, m, l,
+                             out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,87 @@
+// Shared device helpers for the gfx950 kernels: element types, wave and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;                       // raw bfloat16 bits
+
+#define QIL_WAVE 64
+
+// Element type codes of the C interface.
+enum { QIL_F32 = 0, QIL_BF16 = 1 };
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
+
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float ld(const float* p) { return *p; }
+__device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ void st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// Value after a round trip through T (what the reference's cast to the model dtype does).
+template <typename T> __device__ __forceinline__ float round_to(float v);
+template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+
+// Eight consecutive elements as floats.  `aligned` promises 16-byte (bf16) / 32-byte-pair (f32) alignment.
+__device__ __forceinline__ void ld8(const bf16_t* p, float* out) {
+  uint4 raw = *reinterpret_cast<const uint4*>(p);
+  uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __uint_as_float(w[i] << 16);
+    out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void ld8(const float* p, float* out) {
+  float4 a = *reinterpret_cast<const float4*>(p);
+  float4 b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+  out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = QIL_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, QIL_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = QIL_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, QIL_WAVE));
+  return v;
+}
+
+// Block reductions for blocks of up to 16 waves; `scratch` holds 16 floats of LDS.
+// Every thread of the block must call; every thread gets the result.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int waves = (blockDim.x + QIL_WAVE - 1) / QIL_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < waves; ++w) total += scratch[w];      // fixed order
+  return total;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int waves = (blockDim.x + QIL_WAVE - 1) / QIL_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float best = scratch[0];
+  for (int w = 1; w < waves; ++w) best = fmaxf(best, scratch[w]);
+  return best;
+}
+
+// Launch epilogue of every C entry point: 0 on success, the HIP error code otherwise.
+#define QIL_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()

@@ -1,0 +1,71 @@
+"""Trace replay: feed given token ids through the model step by step and write logits.
+
+Nothing is sampled.  The steps go through the same model, step function, cache
+manager and kernels that generation uses.  Input: one JSON object a line,
+``{"step": n, "entries": [{"id": r, "tokens": [...], "want": [...]}, ...], "end": [r, ...]}``.
+For a step that wants something, ``<out>/<step>.f32`` gets the logits at the wanted
+places, in the order of the entries and of ``want``, little-endian float32
+[wanted, vocab].  After every step a line ``done <step>`` is printed and flushed.
+"""
+import argparse
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+from ..weights import load_model
+from .batch import StepEntry
+from .step import ModelRunner
+
+PAGE_SIZE = 16
+ROUND_TO = 64          # a live request's token count is rounded up to this (or to a page, if larger)
+
+
+def pages_for_budget(max_tokens, page_size):
+    unit = -(-ROUND_TO // page_size) * page_size          # 64 rounded up to whole pages
+    return -(-max_tokens // unit) * (unit // page_size)
+
+
+class Replay:
+    def __init__(self, model, *, max_tokens, page_size=PAGE_SIZE, max_requests=64):
+        self.runner = ModelRunner(model, num_pages=pages_for_budget(max_tokens, page_size), page_size=page_size,
+                                  max_requests=max_requests)
+
+    def step(self, record):
+        """Run one parsed step; float32 logits as a CPU array [wanted, vocab] or None."""
+        entries = []
+        for item in record.get('entries', []):
+            request = item['id']
+            if not self.runner.cache.owns(request):
+                if not self.runner.admit(request):
+                    raise RuntimeError(f'no room for another live request ({request!r})')
+            entries.append(StepEntry(request, tuple(item['tokens']), tuple(item.get('want', ()))))
+        logits = self.runner.step(entries) if entries else None
+        for request in record.get('end', []):
+            if self.runner.cache.owns(request):
+                self.runner.release(request)
+        return None if logits is None else logits.to('cpu').numpy()
+
+
+def main(argv=None):
+    parser = argparse.ArgumentParser(prog='trace_run', description=__doc__.splitlines()[0])
+    parser.add_argument('--model', required=True, help='folder with config.json and model.safetensors')
+    parser.add_argument('--dtype', required=True, choices=['bfloat16', 'float32'])
+    parser.add_argument('--out', required=True, type=Path)
+    parser.add_argument('--max-tokens', required=True, type=int,
+                        help='most tokens live requests hold at any time (each rounded up to 64)')
+    args = parser.parse_args(argv)
+    args.out.mkdir(parents=True, exist_ok=True)
+    model = load_model(args.model, dtype=getattr(torch, args.dtype), device='cuda')
+    replay = Replay(model, max_tokens=args.max_tokens)
+    for line in sys.stdin:
+        if not line.strip():
+            continue
+        record = json.loads(line)
+        logits = replay.step(record)
+        if logits is not None:
+            np.ascontiguousarray(logits, dtype='<f4').tofile(args.out / f"{record['step']}.f32")
+        print(f"done {record['step']}", flush=True)
+    return 0

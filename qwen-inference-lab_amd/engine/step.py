@@ -1,0 +1,124 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step may hold portions of prompts beside single decoded tokens, cut anywhere;
+all of it runs as ONE batch over the packed rows (the reference runs each prompt
+portion as a forward of its own and only decode rows together,
+qil/engine.py:59-82).  It runs only the tokens it is given, reads everything
+else from the cache that earlier steps left, and returns float32 logits at the
+wanted places, in entry order.  With nothing wanted, neither the final norm nor
+the head runs (qil/model.py:130-131).
+"""
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from .batch import StepContext, StepEntry
+
+
+class ModelRunner:
+    """Owns the cache of a loaded model and steps batches through it."""
+
+    def __init__(self, model, *, num_pages, page_size=16, max_requests=64, max_step_tokens=None):
+        if not model.loaded:
+            raise ValueError('the model has no weights yet')
+        self.model = model
+        self.max_positions = getattr(model.config, 'max_position_embeddings', None)
+        self.cache = CacheManager(model.cache_needs(), num_pages=num_pages, page_size=page_size,
+                                  max_requests=max_requests, dtype=model.dtype, device=model.device,
+                                  max_step_tokens=max_step_tokens)
+        self.views = self.cache.views()
+        self.steps = 0
+
+    # -- request lifetime (thin: the cache manager decides)
+    def admit(self, request, max_cached_tokens=None):
+        return self.cache.admit(request, max_cached_tokens)
+
+    def release(self, request):
+        self.cache.release(request)
+
+    def computed(self, request):
+        return self.cache.computed[request]
+
+    # -- the step
+    def _validate(self, entries):
+        if not entries:
+            raise ValueError('a step needs at least one entry')
+        seen = set()
+        vocab = self.model.vocab
+        for entry in entries:
+            if entry.request in seen:
+                raise ValueError(f'request {entry.request!r} appears twice in one step')
+            seen.add(entry.request)
+            if not self.cache.owns(entry.request):
+                raise ValueError(f'request {entry.request!r} was not admitted')
+            if not entry.tokens:
+                raise ValueError(f'request {entry.request!r} brings no tokens')
+            if any(type(t) is not int or not 0 <= t < vocab for t in entry.tokens):      # qil/model.py:145-146
+                raise ValueError(f'request {entry.request!r}: token ids must be integers in [0, {vocab})')
+            end = self.cache.computed[entry.request] + len(entry.tokens)
+            if self.max_positions is not None and end > self.max_positions:               # qil/model.py:120
+                raise ValueError(f'request {entry.request!r} would exceed {self.max_positions} positions')
+            if any(type(w) is not int or not 0 <= w < len(entry.tokens) for w in entry.want):
+                raise ValueError(f'request {entry.request!r}: wanted places must index its tokens')
+
+    def prepare(self, entries):
+        """Pages, then the batch description on the device.  Does not touch the cache contents."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2]) if len(e) > 2 else ())
+                   for e in entries]
+        self._validate(entries)
+        cache, ps = self.cache, self.cache.page_size
+        starts = [cache.computed[e.request] for e in entries]
+        for entry, start in zip(entries, starts):
+            cache.ensure(entry.request, start + len(entry.tokens))
+
+        counts = [len(e.tokens) for e in entries]
+        n, s = sum(counts), len(entries)
+        cu = np.zeros(s + 1, dtype=np.int64)
+        cu[1:] = np.cumsum(counts)
+        tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=n)
+        row_seq = np.repeat(np.arange(s), counts)
+        positions = np.arange(n) - cu[row_seq] + np.asarray(starts)[row_seq]
+        logit_rows = np.fromiter((cu[i] + w for i, e in enumerate(entries) for w in e.want), dtype=np.int64)
+        slots = [cache.slots[e.request] for e in entries]
+        max_context = int(max(st + c for st, c in zip(starts, counts)))
+
+        pieces = [tokens, positions, row_seq, cu, np.asarray(starts), np.asarray(slots), logit_rows]
+        group_tables = []
+        for index, group in enumerate(cache.kv_groups):
+            tables = [cache.table(index, e.request) for e in entries]
+            width = max(len(t) for t in tables)
+            table = np.zeros((s, width), dtype=np.int64)
+            for i, t in enumerate(tables):
+                table[i, :len(t)] = t
+            token_slots = table[row_seq, positions // ps] * ps + positions % ps
+            if (table[row_seq, positions // ps] < 0).any():
+                raise RuntimeError('a new token falls into a page that was given back')
+            table[table < 0] = 0          # given-back blocks lie outside every window; never read
+            group_tables.append((width, len(pieces)))
+            pieces += [table.reshape(-1), token_slots]
+        flat = np.concatenate(pieces).astype(np.int32)
+        device = torch.from_numpy(flat).to(self.model.device)
+        offsets = np.cumsum([0] + [len(p) for p in pieces])
+        part = lambda i: device[offsets[i]:offsets[i + 1]]
+
+        ctx = StepContext(
+            n_tokens=n, n_seqs=s, n_logit_rows=len(logit_rows), token_ids=part(0), positions=part(1),
+            row_seq=part(2), cu_seqlens=part(3), seq_starts=part(4), seq_slots=part(5), logit_rows=part(6),
+            max_query=max(counts), max_context=max_context, host_cu_seqlens=cu.tolist(), host_starts=starts,
+            host_slots=slots, requests=[e.request for e in entries])
+        for view in self.views:
+            if view is not None and hasattr(view, 'block_tables'):
+                width, at = group_tables[view.group]
+                view.block_tables = part(at).view(s, width)
+                view.slots = part(at + 1)
+        return entries, ctx
+
+    @torch.inference_mode()
+    def step(self, entries):
+        """Run one batch; float32 logits [wanted, vocab] (None if nothing is wanted)."""
+        entries, ctx = self.prepare(entries)
+        logits = self.model.forward(ctx, self.views)
+        for entry, start in zip(entries, ctx.host_starts):
+            self.cache.advance(entry.request, start + len(entry.tokens))
+        self.steps += 1
+        return logits

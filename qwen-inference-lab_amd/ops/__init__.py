@@ -1,0 +1,232 @@
+"""The kernels as Python functions over torch tensors on the GPU.
+
+Each function checks what its kernel assumes (shapes, types, contiguity, sizes it
+takes), then launches the hand-written HIP kernel on torch's current stream.
+Nothing here computes on the host or through a library, with one exception:
+bfloat16 matrix products with many rows and a bfloat16 result go to the GPU BLAS
+library, where the reference uses one too (nn.Linear, qil/model.py:32-40).  An
+op refuses sizes its kernel does not take with ``UnsupportedShape``; if the
+kernel library cannot be built or loaded every op raises.
+
+Tensors: ``T`` is the model's dtype (float32 or bfloat16).  The residual stream
+is float32.  Index tensors are int32.
+"""
+import torch
+
+from . import library
+
+# Rows up to which a bfloat16 product runs on the weight-streaming kernel whatever its output type.
+STREAM_GEMM_MAX_ROWS = 64
+# Keys per split of the row attention kernel.
+ATTENTION_PART = 256
+
+
+class UnsupportedShape(ValueError):
+    pass
+
+
+_CODES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _code(dtype):
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise UnsupportedShape(f'kernels exist for float32 and bfloat16, not {dtype}') from None
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(tensor):
+    return None if tensor is None else tensor.data_ptr()
+
+
+def _check(status, name):
+    if status:
+        raise RuntimeError(f'{name}: HIP kernel launch failed (status {status})'
+                           if status > 0 else f'{name}: size not taken by the kernel')
+
+
+def _require(tensor, name, dtype=None, shape=None):
+    if not tensor.is_cuda:
+        raise RuntimeError(f'{name} is on {tensor.device}: the kernels run on the GPU only')
+    if not tensor.is_contiguous():
+        raise ValueError(f'{name} must be contiguous')
+    if dtype is not None and tensor.dtype != dtype:
+        raise ValueError(f'{name} must be {dtype}, is {tensor.dtype}')
+    if shape is not None and tuple(tensor.shape) != tuple(shape):
+        raise ValueError(f'{name} must have shape {tuple(shape)}, has {tuple(tensor.shape)}')
+
+
+def check_attention_geometry(*, heads, kv_heads, head_dim, dtype):
+    """Sizes the attention kernels take; called when an attention part is built."""
+    _code(dtype)
+    if heads < 1 or kv_heads < 1 or heads % kv_heads:
+        raise UnsupportedShape(f'heads {heads} must be a positive multiple of kv_heads {kv_heads}')
+    if head_dim % 8 or not 8 <= head_dim <= 256:
+        raise UnsupportedShape(f'head_dim {head_dim}: the attention kernels take multiples of 8 from 8 to 256')
+
+
+def embed(token_ids, table):
+    """int32 [N], T [V, H] -> float32 stream [N, H]."""
+    _require(token_ids, 'token_ids', torch.int32)
+    _require(table, 'table')
+    n, width = token_ids.shape[0], table.shape[1]
+    stream = torch.empty((n, width), dtype=torch.float32, device=table.device)
+    _check(library.load().qil_embed(_ptr(token_ids), _ptr(table), _ptr(stream), n, width, _code(table.dtype),
+                                    _stream()), 'embed')
+    return stream
+
+
+def add_rmsnorm(stream, delta, weight, eps, out_dtype):
+    """stream += delta (in place, float32 sum; skipped if delta is None); returns norm(stream) as out_dtype."""
+    n, width = stream.shape
+    _require(stream, 'stream', torch.float32)
+    _require(weight, 'weight', torch.float32, (width,))
+    if delta is not None:
+        _require(delta, 'delta', out_dtype, (n, width))
+    out = torch.empty((n, width), dtype=out_dtype, device=stream.device)
+    _check(library.load().qil_add_rmsnorm(_ptr(stream), _ptr(delta), None, _ptr(weight), _ptr(out), n, width,
+                                          float(eps), 1, _code(out_dtype), _stream()), 'add_rmsnorm')
+    return out
+
+
+def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
+    """norm(stream[rows] + delta[rows]) as out_dtype [len(rows), H]; stream is left as it is."""
+    n, width = stream.shape
+    _require(stream, 'stream', torch.float32)
+    _require(weight, 'weight', torch.float32, (width,))
+    _require(rows, 'rows', torch.int32)
+    if delta is not None:
+        _require(delta, 'delta', out_dtype, (n, width))
+    out = torch.empty((rows.shape[0], width), dtype=out_dtype, device=stream.device)
+    _check(library.load().qil_add_rmsnorm(_ptr(stream), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out),
+                                          rows.shape[0], width, float(eps), 0, _code(out_dtype), _stream()),
+           'rows_rmsnorm')
+    return out
+
+
+def linear(x, weight, bias=None, out_dtype=None):
+    """x [N, K] @ weight [O, K]^T (+ bias float32 [O]) -> [N, O] in out_dtype (default: x's)."""
+    _require(x, 'x')
+    _require(weight, 'weight', x.dtype)
+    n, k = x.shape
+    o = weight.shape[0]
+    if weight.shape[1] != k:
+        raise ValueError(f'linear: x has {k} columns, weight {weight.shape[1]}')
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, (o,))
+    out_dtype = out_dtype or x.dtype
+    lib = library.load()
+    if x.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise UnsupportedShape('a float32 product has a float32 result')
+        out = torch.empty((n, o), dtype=torch.float32, device=x.device)
+        _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _stream()), 'gemm_f32')
+        return out
+    _code(x.dtype)
+    if out_dtype == torch.float32 or n <= STREAM_GEMM_MAX_ROWS:
+        out = torch.empty((n, o), dtype=out_dtype, device=x.device)
+        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), _stream()),
+               'gemm_bf16')
+        return out
+    out = torch.mm(x, weight.t())                      # GPU BLAS, float32 accumulation
+    if bias is not None:
+        _check(lib.qil_add_bias(_ptr(out), _ptr(bias), n, o, _code(out.dtype), _stream()), 'add_bias')
+    return out
+
+
+def silu_mul(gate_up):
+    """T [N, 2 I] (gate columns first) -> silu(gate) * up, T [N, I]."""
+    _require(gate_up, 'gate_up')
+    n, both = gate_up.shape
+    if both % 2:
+        raise ValueError('silu_mul: needs an even number of columns')
+    out = torch.empty((n, both // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library.load().qil_silu_mul(_ptr(gate_up), _ptr(out), n, both // 2, _code(gate_up.dtype), _stream()),
+           'silu_mul')
+    return out
+
+
+def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
+                       k_cache, v_cache, page_size):
+    """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given); q back
+    into ``qkv`` in place, k and v into the caches at ``slots`` (None: not stored)."""
+    n = qkv.shape[0]
+    _require(qkv, 'qkv', None, (n, (heads + 2 * kv_heads) * head_dim))
+    _require(positions, 'positions', torch.int32, (n,))
+    for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
+        if w is not None:
+            _require(w, name, torch.float32, (head_dim,))
+    if (q_weight is None) != (k_weight is None):
+        raise ValueError('q and k norms come together')
+    cos = sin = None
+    rot = 0
+    if rotation is not None:
+        cos, sin, rot = rotation.cos, rotation.sin, rotation.rot_dim
+        _require(cos, 'cos', torch.float32)
+        _require(sin, 'sin', torch.float32, cos.shape)
+        if cos.shape[1] * 2 != rot or rot > head_dim:
+            raise ValueError('rotation tables do not fit rot_dim')
+    if slots is not None:
+        _require(slots, 'slots', torch.int32, (n,))
+        for cache, name in ((k_cache, 'k_cache'), (v_cache, 'v_cache')):
+            _require(cache, name, qkv.dtype)
+            if cache.ndim != 4 or tuple(cache.shape[1:]) != (kv_heads, page_size, head_dim):
+                raise ValueError(f'{name} must be [pages, {kv_heads}, {page_size}, {head_dim}]')
+    _check(library.load().qil_qk_norm_rope_store(
+        _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots),
+        _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps), _code(qkv.dtype),
+        _stream()), 'qk_norm_rope_store')
+
+
+def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
+                    cu_seqlens, seq_starts, n_seqs, max_query, max_context, scale, window):
+    """Attention of every row of the step over its request's cached keys.
+
+    q is read from the leading ``heads * head_dim`` columns of ``qkv`` [N, (heads + 2 kv_heads) d].
+    Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
+    j <= positions[n] and, with a window, j > positions[n] - window.  -> T [N, heads * head_dim].
+    """
+    n = qkv.shape[0]
+    check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=head_dim, dtype=qkv.dtype)
+    _require(qkv, 'qkv', None, (n, (heads + 2 * kv_heads) * head_dim))
+    _require(block_tables, 'block_tables', torch.int32)
+    _require(row_seq, 'row_seq', torch.int32, (n,))
+    _require(positions, 'positions', torch.int32, (n,))
+    for cache, name in ((k_cache, 'k_cache'), (v_cache, 'v_cache')):
+        _require(cache, name, qkv.dtype)
+        if cache.ndim != 4 or tuple(cache.shape[1:]) != (kv_heads, page_size, head_dim):
+            raise ValueError(f'{name} must be [pages, {kv_heads}, {page_size}, {head_dim}]')
+    if block_tables.ndim != 2 or block_tables.shape[1] * page_size < max_context:
+        raise ValueError('block_tables are too narrow for the longest context')
+    lib = library.load()
+    part = ATTENTION_PART
+    parts = max(1, -(-max_context // part))
+    out = torch.empty((n, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    nbytes = lib.qil_attn_rows_workspace(n, heads, head_dim, parts)
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
+    _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                             block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(workspace), _ptr(out), n,
+                             heads, kv_heads, head_dim, page_size, int(window or 0), float(scale), part, parts,
+                             _code(qkv.dtype), _stream()), 'attn_rows')
+    return out
+
+
+def sample(logits, temperatures, seeds, counters):
+    """float32 [M, V] -> (int32 tokens [M], int32 finite flags [M]).
+
+    temperature 0: greedy, lowest index on ties; > 0: seeded Gumbel-max draw from softmax(logits / T)
+    keyed by (seed, counter)."""
+    m, vocab = logits.shape
+    _require(logits, 'logits', torch.float32)
+    _require(temperatures, 'temperatures', torch.float32, (m,))
+    _require(seeds, 'seeds', torch.int32, (m,))
+    _require(counters, 'counters', torch.int32, (m,))
+    tokens = torch.empty(m, dtype=torch.int32, device=logits.device)
+    finite = torch.empty(m, dtype=torch.int32, device=logits.device)
+    _check(library.load().qil_sample(_ptr(logits), _ptr(temperatures), _ptr(seeds), _ptr(counters), _ptr(tokens),
+                                     _ptr(finite), m, vocab, _stream()), 'sample')
+    return tokens, finite

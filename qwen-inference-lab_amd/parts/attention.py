@@ -1,0 +1,72 @@
+"""Grouped-query attention over the paged cache.  Formulas: qil/model.py:48-69, :73-84."""
+import torch
+
+from .base import Mixer, ParamSpec, KVNeed
+from .. import ops
+
+
+class Attention(Mixer):
+    """q/k/v projections (+bias), optional per-head RMSNorm of q and k, position
+    encoding, write of k/v into the request's pages, attention of the step's
+    queries over everything cached (key j visible iff j <= position, and
+    j > position - window if a window is set), output projection (+bias).
+
+    Query head h reads kv head h // (heads / kv_heads)  (qil/model.py:59-61).
+    The three projection matrices are stacked at ``finalize`` into one
+    [(heads + 2 kv_heads) head_dim, width] matrix: a pure re-layout, each output
+    column is computed from the same row as before.
+    """
+
+    def __init__(self, *, width, heads, kv_heads, head_dim, bias, qk_norm_eps, scale,
+                 position=None, window=None, dtype=torch.bfloat16):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError('heads must be a multiple of kv_heads')
+        self.width, self.heads, self.kv_heads, self.head_dim = width, heads, kv_heads, head_dim
+        self.bias, self.qk_norm_eps, self.scale = bool(bias), qk_norm_eps, float(scale)
+        self.position, self.window, self.dtype = position, window, dtype
+        ops.check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=head_dim, dtype=dtype)
+
+    def param_specs(self):
+        q, kv, d = self.heads * self.head_dim, self.kv_heads * self.head_dim, self.head_dim
+        specs = {'q_proj.weight': ParamSpec((q, self.width)), 'k_proj.weight': ParamSpec((kv, self.width)),
+                 'v_proj.weight': ParamSpec((kv, self.width)), 'o_proj.weight': ParamSpec((self.width, q))}
+        if self.bias:   # o_proj gets a bias too (qil/model.py:35)
+            specs.update({'q_proj.bias': ParamSpec((q,), 'vector'), 'k_proj.bias': ParamSpec((kv,), 'vector'),
+                          'v_proj.bias': ParamSpec((kv,), 'vector'), 'o_proj.bias': ParamSpec((self.width,), 'vector')})
+        if self.qk_norm_eps is not None:
+            specs.update({'q_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal'),
+                          'k_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal')})
+        return specs
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.head_dim, self.window)
+
+    def finalize(self):
+        p = self.p
+        self.w_qkv = torch.cat([p.pop('q_proj.weight'), p.pop('k_proj.weight'), p.pop('v_proj.weight')]).contiguous()
+        self.b_qkv = (torch.cat([p.pop('q_proj.bias'), p.pop('k_proj.bias'), p.pop('v_proj.bias')]).contiguous()
+                      if self.bias else None)
+        p['qkv_proj.weight'] = self.w_qkv
+        if self.bias:
+            p['qkv_proj.bias'] = self.b_qkv
+
+    def forward(self, h, ctx, cache):
+        p = self.p
+        qkv = ops.linear(h, self.w_qkv, self.b_qkv)
+        rotation = self.position.rotation() if self.position is not None else None
+        ops.qk_norm_rope_store(
+            qkv, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
+            q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
+            eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+            rotation=rotation, positions=ctx.positions,
+            slots=cache.slots if cache.writes else None,
+            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size)
+        attended = ops.paged_attention(
+            qkv, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
+            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
+            block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
+            cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, n_seqs=ctx.n_seqs,
+            max_query=ctx.max_query, max_context=ctx.max_context,
+            scale=self.scale, window=self.window)
+        return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'))

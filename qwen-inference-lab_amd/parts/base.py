@@ -1,0 +1,132 @@
+"""What every part is: a holder of declared tensors with a forward of its kind.
+
+A part never learns which model it sits in.  It receives its sizes and constants
+as constructor arguments, declares its tensors in ``param_specs()``, gets them
+through ``set_param`` (from a checkpoint or a random generator), may re-lay them
+out once in ``finalize()``, and computes with the kernels of ``qil_amd.ops``.
+
+Tensor kinds (``ParamSpec.kind``):
+  matrix  -> stored in the model's dtype (bfloat16 or float32)
+  vector  -> norm scales and biases; always float32 on the device, which holds a
+             bfloat16 or a float32 checkpoint value exactly
+  table   -> integer tables; int32
+"""
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: tuple
+    kind: str = 'matrix'          # matrix | vector | table
+    init: str = 'normal'          # normal | one_plus_normal | zeros
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Per-token keys and values in pages.  ``window`` None keeps every key."""
+    kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Fixed-size per-request state, one slot per live request.
+
+    dtype: 'float32' or 'model'.  The slot of a request that starts (start == 0)
+    must be treated as empty by the mixer; the cache manager does not clear it.
+    """
+    shape: tuple
+    dtype: str = 'float32'
+
+
+class Part:
+    def __init__(self):
+        self.p = {}
+
+    def param_specs(self):
+        """dict local name -> ParamSpec."""
+        return {}
+
+    def set_param(self, name, tensor):
+        spec = self.param_specs()[name]
+        if tuple(tensor.shape) != tuple(spec.shape):
+            raise ValueError(f'{type(self).__name__}.{name}: shape {tuple(tensor.shape)} != {tuple(spec.shape)}')
+        self.p[name] = tensor
+
+    def finalize(self):
+        """Called once after every declared tensor is set."""
+
+    def parameter_bytes(self):
+        return sum(t.numel() * t.element_size() for t in self.p.values())
+
+
+class Norm(Part):
+    """[N, width] float32 stream -> normalised [N, width] in ``out_dtype``.
+
+    ``forward(stream, delta, out_dtype)``: if ``delta`` is given it is first added
+    into ``stream`` in place (float32 sum), then the sum is normalised.
+    ``forward_rows(stream, delta, rows, out_dtype)``: the same for the selected
+    rows only, leaving ``stream`` untouched.
+    """
+    def forward(self, stream, delta, out_dtype):
+        raise NotImplementedError
+
+    def forward_rows(self, stream, delta, rows, out_dtype):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Something the mixer applies to queries and keys by absolute position.
+
+    ``rotation()`` returns None (nothing to apply) or a ``Rotation`` record that
+    the fused query/key kernel understands.
+    """
+    def rotation(self):
+        return None
+
+
+@dataclass(frozen=True)
+class Rotation:
+    cos: object            # float32 [positions, rot_dim/2]
+    sin: object
+    rot_dim: int           # leading rot_dim elements of each head are rotated, pairs (i, i + rot_dim/2)
+
+
+class Mixer(Part):
+    """Token mixer: [N, width] -> [N, width] over the step's batch and the cache.
+
+    ``cache_need()`` says what it keeps between steps (KVNeed, StateNeed or None);
+    ``forward(h, ctx, cache)`` gets the step context (engine/batch.py) and the
+    cache view of its schedule entry (cache/manager.py: KVView or StateView).
+    Its result must not depend on how a request's tokens were cut into steps.
+    """
+    def cache_need(self):
+        return None
+
+    def forward(self, h, ctx, cache):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Per-token map [N, width] -> [N, width]."""
+    def forward(self, h):
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of parts around the residual stream.
+
+    ``forward(stream, pending, ctx, cache)`` -> pending: ``stream`` is the float32
+    residual stream [N, width], changed in place; ``pending`` is a sub-layer
+    output not yet added to it (or None), which lets the add fuse into the next
+    norm.  The block returns its own last sub-layer output as the new pending.
+    """
+    mixer = None
+
+    def parts(self):
+        """dict local prefix -> Part (for naming tensors)."""
+        return {}
+
+    def forward(self, stream, pending, ctx, cache):
+        raise NotImplementedError

@@ -1,0 +1,30 @@
+"""Gated feed-forward: down(act(gate(x)) * up(x)).  Formula: qil/model.py:71."""
+import torch
+
+from .base import FeedForward, ParamSpec
+from .. import ops
+
+
+class GatedMLP(FeedForward):
+    """``activation`` names the gate's function; 'silu' (z * sigmoid(z)) is the one
+    the kernels have.  Gate and up matrices are stacked at ``finalize`` into one
+    [2 * intermediate, width] matrix (gate rows first): a pure re-layout."""
+
+    def __init__(self, *, width, intermediate, activation='silu'):
+        super().__init__()
+        if activation != 'silu':
+            raise ValueError(f'no kernel for activation {activation!r}')
+        self.width, self.intermediate, self.activation = width, intermediate, activation
+
+    def param_specs(self):
+        return {'gate_proj.weight': ParamSpec((self.intermediate, self.width)),
+                'up_proj.weight': ParamSpec((self.intermediate, self.width)),
+                'down_proj.weight': ParamSpec((self.width, self.intermediate))}
+
+    def finalize(self):
+        p = self.p
+        p['gate_up_proj.weight'] = torch.cat([p.pop('gate_proj.weight'), p.pop('up_proj.weight')]).contiguous()
+
+    def forward(self, h):
+        gate_up = ops.linear(h, self.p['gate_up_proj.weight'], None)
+        return ops.linear(ops.silu_mul(gate_up), self.p['down_proj.weight'], None)

@@ -1,0 +1,4 @@
+"""Sampling."""
+from .sampler import Sampler, SamplingParams
+
+__all__ = ['Sampler', 'SamplingParams']

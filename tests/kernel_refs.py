@@ -1,0 +1,125 @@
+"""Plain torch references of the HIP kernels, one per op of ``qil_amd.ops``, same signatures.
+
+Two uses: GPU tests compare each kernel with its reference here; CPU tests
+substitute these for the kernels (pytest monkeypatch) to exercise the cache
+manager, the step function, the scheduler and trace replay without a GPU.  They
+are test code: the engine never imports them.
+"""
+import torch
+
+
+def _round(x, dtype):
+    return x.to(dtype).to(torch.float32)
+
+
+def embed(token_ids, table):
+    return table[token_ids.long()].to(torch.float32)
+
+
+def _norm(x, weight, eps, out_dtype):
+    n = x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + eps)
+    return (_round(n, out_dtype) * weight).to(out_dtype)
+
+
+def add_rmsnorm(stream, delta, weight, eps, out_dtype):
+    if delta is not None:
+        stream += delta.to(torch.float32)
+    return _norm(stream, weight, eps, out_dtype)
+
+
+def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
+    x = stream[rows.long()]
+    if delta is not None:
+        x = x + delta[rows.long()].to(torch.float32)
+    return _norm(x, weight, eps, out_dtype)
+
+
+def linear(x, weight, bias=None, out_dtype=None):
+    y = x.to(torch.float32) @ weight.to(torch.float32).t()
+    if bias is not None:
+        y = y + bias
+    return y.to(out_dtype or x.dtype)
+
+
+def silu_mul(gate_up):
+    inner = gate_up.shape[1] // 2
+    g, u = gate_up[:, :inner].to(torch.float32), gate_up[:, inner:].to(torch.float32)
+    return (g / (1 + torch.exp(-g)) * u).to(gate_up.dtype)
+
+
+def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
+                       k_cache, v_cache, page_size):
+    n, d = qkv.shape[0], head_dim
+    x = qkv.view(n, heads + 2 * kv_heads, d)
+    q, k, v = x[:, :heads].to(torch.float32), x[:, heads:heads + kv_heads].to(torch.float32), x[:, heads + kv_heads:]
+
+    def shape(t, weight):
+        if weight is not None:
+            t = _round(t * torch.rsqrt(t.square().mean(dim=-1, keepdim=True) + eps), qkv.dtype) * weight
+        if rotation is not None:
+            rot, half = rotation.rot_dim, rotation.rot_dim // 2
+            c = rotation.cos[positions.long()][:, None, :]
+            s = rotation.sin[positions.long()][:, None, :]
+            left, right = t[..., :half], t[..., half:rot]
+            t = torch.cat((left * c - right * s, left * s + right * c, t[..., rot:]), dim=-1)
+        return t.to(qkv.dtype)
+
+    x[:, :heads] = shape(q, q_weight)
+    if slots is not None:
+        page, offset = slots.long() // page_size, slots.long() % page_size
+        k_cache[page, :, offset] = shape(k, k_weight)
+        v_cache[page, :, offset] = v
+
+
+def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
+                    cu_seqlens, seq_starts, n_seqs, max_query, max_context, scale, window, accumulate=torch.float32):
+    n, d, g = qkv.shape[0], head_dim, heads // kv_heads
+    q = qkv[:, :heads * d].reshape(n, heads, d).to(accumulate)
+    out = torch.empty((n, heads, d), dtype=accumulate, device=qkv.device)
+    for row in range(n):
+        ctx = int(positions[row]) + 1
+        lo = max(0, ctx - window) if window else 0
+        j = torch.arange(lo, ctx, device=qkv.device)
+        pages = block_tables[int(row_seq[row])].long()[j // page_size]
+        keys = k_cache[pages, :, j % page_size].to(accumulate)          # [ctx, kv_heads, d]
+        values = v_cache[pages, :, j % page_size].to(accumulate)
+        keys = keys.repeat_interleave(g, dim=1)
+        values = values.repeat_interleave(g, dim=1)
+        scores = torch.einsum('hd,jhd->hj', q[row], keys) * scale
+        out[row] = torch.einsum('hj,jhd->hd', torch.softmax(scores, dim=-1), values)
+    return out.reshape(n, heads * d).to(qkv.dtype)
+
+
+def _uniform(seed, counter, vocab, device):
+    i = torch.arange(vocab, dtype=torch.int64, device=device)
+    offset = (((int(seed) & 0xFFFFFFFF) * 0x85EBCA77) + ((int(counter) & 0xFFFFFFFF) * 0xC2B2AE3D)) & 0xFFFFFFFF
+    x = (i * 0x9E3779B1 + offset) & 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return ((x >> 8).to(torch.float32) + 0.5) * (1.0 / 16777216.0)
+
+
+def sample_scores(logits, temperatures, seeds, counters):
+    """The perturbed scores whose argmax is the draw (plain logits for temperature 0)."""
+    rows = []
+    for r in range(logits.shape[0]):
+        t = float(temperatures[r])
+        if t > 0:
+            u = _uniform(int(seeds[r]), int(counters[r]), logits.shape[1], logits.device)
+            rows.append(logits[r] / t - torch.log(-torch.log(u)))
+        else:
+            rows.append(logits[r])
+    return torch.stack(rows)
+
+
+def sample(logits, temperatures, seeds, counters):
+    scores = sample_scores(logits, temperatures, seeds, counters)
+    finite = torch.isfinite(logits).all(dim=-1).to(torch.int32)
+    return scores.argmax(dim=-1).to(torch.int32), finite
+
+
+ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, silu_mul=silu_mul,
+           qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample)

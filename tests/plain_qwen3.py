@@ -1,0 +1,275 @@
+"""Plain, slow Qwen3-dense implementation used as the oracle of every test.
+
+Whole sequences, no cache, no batching, one function per part, torch CPU
+tensors only.  Nothing here imports the engine; the engine imports nothing from
+here.  Each function cites the reference lines (relative to the reference
+repository root) whose formula it restates.
+
+`weights` is a dict from checkpoint tensor names to tensors; `config` is the
+dict of config.json.  `dtype` is the arithmetic type: float32 (default),
+float64 for tight pins, or bfloat16 to follow the reference's rounding places.
+"""
+import math
+
+import torch
+
+
+# --------------------------------------------------------------------------- parts
+
+def inverse_frequencies(head_dim, theta):
+    """inv_freq[i] = 1 / theta**(2i/d), i < d/2, in float32 on the CPU.
+
+    qil/model.py:103-104 (positive exponent, then reciprocal; never theta**(-e)).
+    """
+    exponent = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
+    return 1.0 / (theta ** exponent)
+
+
+def rotary_angles(positions, head_dim, theta):
+    """angle[t, i] = float32(position[t]) * inv_freq[i].  qil/model.py:106-108."""
+    return positions.to(torch.float32)[:, None] * inverse_frequencies(head_dim, theta)[None, :]
+
+
+def rotate(x, angles):
+    """Split-half rotation of x[T, heads, d] by angles[T, d/2].
+
+    out = concat(left*cos - right*sin, left*sin + right*cos), the pair being
+    (i, i + d/2); cos and sin are cast to x's type first.  qil/model.py:42-46.
+    """
+    cosine = angles.cos().to(x.dtype)[:, None, :]
+    sine = angles.sin().to(x.dtype)[:, None, :]
+    half = x.shape[-1] // 2
+    left, right = x[..., :half], x[..., half:]
+    return torch.cat((left * cosine - right * sine, left * sine + right * cosine), dim=-1)
+
+
+def rms_norm(x, weight, eps):
+    """y = cast(x32 * rsqrt(mean(x32^2) + eps)) * weight.  qil/model.py:15-23.
+
+    Statistics in float32 (float64 if x is float64); the cast back to x's type
+    comes before the multiplication by the weight; the weight multiplies as it
+    is (no 1 + w).
+    """
+    wide = x.to(torch.float64 if x.dtype == torch.float64 else torch.float32)
+    normalized = wide * (wide.square().mean(dim=-1, keepdim=True) + eps).rsqrt()
+    return normalized.to(x.dtype) * weight
+
+
+def linear(x, weight, bias=None):
+    """y = x W^T (+ b), W stored [out, in].  qil/model.py:32-40 (nn.Linear)."""
+    y = x @ weight.transpose(0, 1)
+    return y if bias is None else y + bias
+
+
+def expand_kv(t, group):
+    """[T, nkv, d] -> [T, nkv*group, d]: query head h reads kv head h // group.
+
+    qil/model.py:59-61 (repeat_interleave), qil/paged_attention.py:25.
+    """
+    T, nkv, d = t.shape
+    return t[:, :, None, :].expand(T, nkv, group, d).reshape(T, nkv * group, d)
+
+
+def attention(q, k, v, positions, scale, window=None):
+    """Masked softmax attention with explicit scores.
+
+    q[T, nq, d] at absolute `positions[T]`; k, v[E, nkv, d] hold positions 0..E-1.
+    score[h, t, j] = q[t, h] . k[j, h // g] * scale; key j is visible to query t
+    iff j <= position[t] (absolute positions, qil/model.py:62-64); softmax over j;
+    out[t, h] = sum_j P[h, t, j] v[j, h // g].  qil/model.py:59-68; scale :67.
+    `window` (not part of Qwen3 dense; for tests of the windowed kernel) hides
+    keys with j <= position[t] - window.
+    """
+    T, nq, d = q.shape
+    E, nkv, _ = k.shape
+    group = nq // nkv
+    kh = expand_kv(k, group).permute(1, 0, 2)            # [nq, E, d]
+    vh = expand_kv(v, group).permute(1, 0, 2)
+    qh = q.permute(1, 0, 2)                              # [nq, T, d]
+    acc = torch.float64 if q.dtype == torch.float64 else torch.float32
+    scores = (qh.to(acc) @ kh.to(acc).transpose(1, 2)) * scale
+    columns = torch.arange(E)[None, :]
+    visible = columns <= positions[:, None]
+    if window is not None:
+        visible = visible & (columns > positions[:, None] - window)
+    scores = scores.masked_fill(~visible[None], float('-inf'))
+    probabilities = torch.softmax(scores, dim=-1)
+    out = probabilities @ vh.to(acc)                     # [nq, T, d]
+    return out.permute(1, 0, 2).to(q.dtype)
+
+
+def attention_block(x, weights, prefix, config, positions):
+    """x + o_proj(attention(rope(qnorm(q)), rope(knorm(k)), v)).  qil/model.py:48-69."""
+    nq, nkv, d = config['num_attention_heads'], config['num_key_value_heads'], config['head_dim']
+    eps = config.get('rms_norm_eps', 1e-6)                         # qil/config.py:18
+    theta = config.get('rope_theta', 1000000.)                     # qil/config.py:19
+    T = x.shape[0]
+    n = rms_norm(x, weights[prefix + 'input_layernorm.weight'], eps)          # :51
+    a = prefix + 'self_attn.'
+    q = linear(n, weights[a + 'q_proj.weight'], weights.get(a + 'q_proj.bias')).reshape(T, nq, d)
+    k = linear(n, weights[a + 'k_proj.weight'], weights.get(a + 'k_proj.bias')).reshape(T, nkv, d)
+    v = linear(n, weights[a + 'v_proj.weight'], weights.get(a + 'v_proj.bias')).reshape(T, nkv, d)
+    q = rms_norm(q, weights[a + 'q_norm.weight'], eps)                         # :52
+    k = rms_norm(k, weights[a + 'k_norm.weight'], eps)                         # :53
+    angles = rotary_angles(positions, d, theta)
+    q, k = rotate(q, angles), rotate(k, angles)                                # :55
+    attended = attention(q, k, v, positions, d ** -0.5).reshape(T, nq * d)     # :65-68
+    return x + linear(attended, weights[a + 'o_proj.weight'], weights.get(a + 'o_proj.bias'))
+
+
+def gated_mlp(n, gate, up, down):
+    """down(silu(gate(n)) * up(n)), silu(z) = z * sigmoid(z).  qil/model.py:71."""
+    g = linear(n, gate)
+    return linear((g * torch.sigmoid(g)) * linear(n, up), down)
+
+
+def mlp_block(x, weights, prefix, config):
+    """x + mlp(norm(x)).  qil/model.py:70-71."""
+    n = rms_norm(x, weights[prefix + 'post_attention_layernorm.weight'], config.get('rms_norm_eps', 1e-6))
+    m = prefix + 'mlp.'
+    return x + gated_mlp(n, weights[m + 'gate_proj.weight'], weights[m + 'up_proj.weight'],
+                         weights[m + 'down_proj.weight'])
+
+
+def decoder_layer(x, weights, index, config, positions):
+    """Pre-norm block: attention then MLP, each added to the stream.  qil/model.py:48-71."""
+    prefix = f'model.layers.{index}.'
+    x = attention_block(x, weights, prefix, config, positions)
+    return mlp_block(x, weights, prefix, config)
+
+
+def head_weight(weights, config):
+    """Tied head shares the embedding (default when the key is absent).
+
+    qil/model.py:96-98, qil/config.py:21.
+    """
+    if config.get('tie_word_embeddings', True):
+        return weights['model.embed_tokens.weight']
+    return weights['lm_head.weight']
+
+
+# --------------------------------------------------------------------------- whole model
+
+def cast_weights(weights, dtype):
+    return {name: t.to(dtype) for name, t in weights.items()}
+
+
+def hidden_states(tokens, weights, config, start=0):
+    """Final hidden states (before the last norm) of one whole sequence.  qil/model.py:123-129."""
+    tokens = torch.as_tensor(tokens, dtype=torch.long)
+    positions = torch.arange(start, start + len(tokens))
+    x = weights['model.embed_tokens.weight'][tokens]                           # :126, no scaling
+    for index in range(config['num_hidden_layers']):
+        x = decoder_layer(x, weights, index, config, positions)
+    return x
+
+
+def logits(tokens, weights, config, dtype=torch.float32):
+    """float32 logits [T, V] at every position of one sequence.  qil/model.py:110-134."""
+    w = cast_weights(weights, dtype)
+    x = hidden_states(tokens, w, config)
+    n = rms_norm(x, w['model.norm.weight'], config.get('rms_norm_eps', 1e-6))
+    return linear(n, head_weight(w, config)).to(torch.float32)                 # :134
+
+
+def greedy(prompt, count, weights, config, dtype=torch.float32):
+    """Full-recompute greedy continuation; ties take the lowest index.  qil/engine.py:96-100."""
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(logits(tokens, weights, config, dtype)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+# --------------------------------------------------------------------------- sampling
+
+def gumbel_uniform(seed, index, vocab):
+    """The sampler's counter-based uniforms, restated on the host (no reference analogue).
+
+    u[i] in (0, 1) from a 32-bit mix of (seed, output index, vocabulary index).
+    """
+    i = torch.arange(vocab, dtype=torch.int64)
+    offset = (((int(seed) & 0xFFFFFFFF) * 0x85EBCA77) + ((int(index) & 0xFFFFFFFF) * 0xC2B2AE3D)) & 0xFFFFFFFF
+    x = (i * 0x9E3779B1 + offset) & 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return ((x >> 8).to(torch.float32) + 0.5) * (1.0 / 16777216.0)
+
+
+def sample(row, temperature, seed, index):
+    """Greedy if temperature == 0 else Gumbel-max draw from softmax(row / T).
+
+    Returns (token, perturbed scores) so a caller can check margins.
+    """
+    row = row.to(torch.float32)
+    if not torch.isfinite(row).all():                                          # qil/engine.py:97-98
+        raise RuntimeError('non-finite logits')
+    if temperature == 0:
+        return int(row.argmax()), row
+    u = gumbel_uniform(seed, index, row.numel())
+    scores = row / temperature - torch.log(-torch.log(u))
+    return int(scores.argmax()), scores
+
+
+# --------------------------------------------------------------------------- random weights
+
+def tensor_shapes(config):
+    """Checkpoint names and shapes of Qwen3 dense.  qil/model.py:159-176, :32-40."""
+    H, I = config['hidden_size'], config['intermediate_size']
+    nq, nkv, d = config['num_attention_heads'], config['num_key_value_heads'], config['head_dim']
+    shapes = {'model.embed_tokens.weight': (config['vocab_size'], H)}
+    for i in range(config['num_hidden_layers']):
+        p = f'model.layers.{i}.'
+        shapes[p + 'input_layernorm.weight'] = (H,)
+        for name, out in (('q_proj', nq * d), ('k_proj', nkv * d), ('v_proj', nkv * d)):
+            shapes[p + f'self_attn.{name}.weight'] = (out, H)
+            if config.get('attention_bias', False):
+                shapes[p + f'self_attn.{name}.bias'] = (out,)
+        shapes[p + 'self_attn.o_proj.weight'] = (H, nq * d)
+        if config.get('attention_bias', False):
+            shapes[p + 'self_attn.o_proj.bias'] = (H,)                         # :35, o_proj too
+        shapes[p + 'self_attn.q_norm.weight'] = (d,)
+        shapes[p + 'self_attn.k_norm.weight'] = (d,)
+        shapes[p + 'post_attention_layernorm.weight'] = (H,)
+        shapes[p + 'mlp.gate_proj.weight'] = (I, H)
+        shapes[p + 'mlp.up_proj.weight'] = (I, H)
+        shapes[p + 'mlp.down_proj.weight'] = (H, I)
+    shapes['model.norm.weight'] = (H,)
+    if not config.get('tie_word_embeddings', True):
+        shapes['lm_head.weight'] = (config['vocab_size'], H)
+    return shapes
+
+
+def random_weights(config, seed, std=0.02, norm_std=0.01, round_to=torch.bfloat16):
+    """Test weights of the plain implementation's own making (not the engine's generator).
+
+    Matrices N(0, std), norm weights 1 + N(0, norm_std); values are rounded to
+    `round_to` and returned as float32 so that both precisions share them exactly.
+    """
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(config).items():
+        t = torch.randn(shape, generator=g, dtype=torch.float32)
+        t = 1.0 + norm_std * t if name.endswith('norm.weight') or name.endswith('layernorm.weight') else std * t
+        out[name] = t.to(round_to).to(torch.float32) if round_to is not None else t
+    return out
+
+
+TINY_A = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=256, hidden_size=64,
+              intermediate_size=128, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=16, max_position_embeddings=512, rms_norm_eps=1e-6, rope_theta=10000.0,
+              attention_bias=False, tie_word_embeddings=True, hidden_act='silu', eos_token_id=None)
+
+TINY_B = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=384, hidden_size=96,
+              intermediate_size=224, num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=2,
+              head_dim=32, max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=1000000.0,
+              attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=[7, 9])
+
+# A third variant: biases on q/k/v/o, sizes that are neither powers of two nor multiples of 32,
+# an odd vocabulary, MQA-like grouping.
+TINY_C = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=301, hidden_size=72,
+              intermediate_size=136, num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=1,
+              head_dim=48, max_position_embeddings=640, rms_norm_eps=3e-6, rope_theta=50000.0,
+              attention_bias=True, tie_word_embeddings=False, hidden_act='silu', eos_token_id=3)

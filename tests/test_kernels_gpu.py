@@ -1,0 +1,328 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the tiny models'."""
+import pytest
+import torch
+
+import kernel_refs as refs
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: dict(atol=2e-6, rtol=2e-5), torch.bfloat16: dict(atol=0.008, rtol=0.008)}
+
+
+@pytest.fixture(scope='module')
+def ops():
+    from qil_amd import ops
+    ops.library.load()
+    return ops
+
+
+def rand(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+def check(actual, expected, dtype, scale=1.0):
+    assert torch.isfinite(actual.float()).all()
+    tol = {k: v * (scale if k == 'atol' else 1) for k, v in TOL[dtype].items()}
+    torch.testing.assert_close(actual.float().cpu(), expected.float().cpu(), **tol)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('vocab,width', [(301, 72), (1000, 1024), (50, 4100)])
+def test_embed(ops, dtype, vocab, width):
+    table = rand(vocab, width, dtype=dtype)
+    tokens = torch.tensor([0, vocab - 1, 7, 7, vocab // 2], dtype=torch.int32).cuda()
+    out = ops.embed(tokens, table)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out, table[tokens.long()].float(), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('rows,width', [(1, 72), (5, 1000), (3, 4096), (2, 5120)])
+def test_add_rmsnorm(ops, dtype, rows, width):
+    stream, delta = rand(rows, width, scale=3.0), rand(rows, width, dtype=dtype, seed=1)
+    weight = (1 + 0.3 * rand(width, seed=2)).contiguous()
+    for eps in (1e-6, 1e-2):
+        want_stream = stream.clone()
+        want = refs.add_rmsnorm(want_stream, delta, weight, eps, dtype)
+        got_stream = stream.clone()
+        got = ops.add_rmsnorm(got_stream, delta, weight, eps, dtype)
+        torch.testing.assert_close(got_stream, want_stream, atol=0, rtol=0)
+        check(got, want, dtype, scale=4)
+        check(ops.add_rmsnorm(got_stream.clone(), None, weight, eps, dtype),
+              refs.add_rmsnorm(want_stream.clone(), None, weight, eps, dtype), dtype, scale=4)
+    # a library routine pins the formula: float32, no delta
+    if dtype == torch.float32:
+        expected = torch.nn.functional.rms_norm(stream, (width,), weight, 1e-6)
+        check(ops.add_rmsnorm(stream.clone(), None, weight, 1e-6, dtype), expected, dtype, scale=4)
+    rows_index = torch.tensor([rows - 1, 0], dtype=torch.int32).cuda()
+    before = stream.clone()
+    got = ops.rows_rmsnorm(stream, delta, rows_index, weight, 1e-5, dtype)
+    torch.testing.assert_close(stream, before, atol=0, rtol=0)
+    check(got, refs.rows_rmsnorm(stream, delta, rows_index, weight, 1e-5, dtype), dtype, scale=4)
+
+
+def test_rmsnorm_rounds_before_the_weight(ops):
+    """bfloat16: the normalised value is rounded, then multiplied by the weight (qil/model.py:22-23)."""
+    width = 64
+    stream = rand(1, width, scale=2.0)
+    weight = torch.full((width,), 1.00390625 + 2 ** -10).cuda()      # not a bfloat16 number
+    got = ops.add_rmsnorm(stream.clone(), None, weight, 1e-6, torch.bfloat16).float()
+    n = stream * torch.rsqrt(stream.square().mean(-1, keepdim=True) + 1e-6)
+    rounded_first = (n.bfloat16().float() * weight).bfloat16().float()
+    torch.testing.assert_close(got, rounded_first, atol=0, rtol=0)
+
+
+SHAPES = [(1, 301, 72), (5, 384, 96), (17, 200, 136), (70, 130, 52), (130, 257, 1030), (8, 4096, 4096),
+          (64, 1000, 2048), (33, 96, 224), (300, 192, 96)]
+
+
+@pytest.mark.parametrize('m,n,k', SHAPES)
+@pytest.mark.parametrize('bias', [False, True])
+def test_linear_float32(ops, m, n, k, bias):
+    x, w = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5)
+    b = rand(n, seed=2) if bias else None
+    want = (x.double() @ w.double().t() + (b.double() if bias else 0)).float()
+    check(ops.linear(x, w, b), want, torch.float32, scale=4)
+
+
+@pytest.mark.parametrize('m,n,k', SHAPES)
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('bias', [False, True])
+def test_linear_bfloat16(ops, m, n, k, out_dtype, bias):
+    x, w = rand(m, k, dtype=torch.bfloat16), rand(n, k, dtype=torch.bfloat16, seed=1, scale=k ** -0.5)
+    b = rand(n, seed=2) if bias else None
+    want = x.double() @ w.double().t() + (b.double() if bias else 0)
+    got = ops.linear(x, w, b, out_dtype=out_dtype)
+    assert got.dtype == out_dtype
+    if out_dtype == torch.float32:           # exact products, float32 sums: only the order differs
+        check(got, want, torch.float32, scale=8)
+    else:
+        check(got, want, torch.bfloat16, scale=2)
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops):
+    """A row's result is the same alone, among 7 and among 40 (same kernel family): bit for bit."""
+    x, w = rand(40, 512, dtype=torch.bfloat16), rand(300, 512, dtype=torch.bfloat16, seed=1, scale=0.05)
+    whole = ops.linear(x, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(ops.linear(x[3:4].contiguous(), w, None, out_dtype=torch.float32), whole[3:4], atol=0, rtol=0)
+    torch.testing.assert_close(ops.linear(x[:7].contiguous(), w, None, out_dtype=torch.float32), whole[:7], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_silu_mul(ops, dtype):
+    gate_up = rand(7, 2 * 136, dtype=dtype, scale=3.0)
+    want = torch.nn.functional.silu(gate_up[:, :136].double()) * gate_up[:, 136:].double()
+    check(ops.silu_mul(gate_up), want, dtype, scale=8)
+
+
+class Rot:
+    def __init__(self, head_dim, theta, positions, rot_dim=None):
+        rot_dim = rot_dim or head_dim
+        angles = plain.rotary_angles(torch.arange(positions), rot_dim, theta)
+        self.cos, self.sin, self.rot_dim = angles.cos().cuda(), angles.sin().cuda(), rot_dim
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('heads,kv_heads,d,rot,page_size', [(4, 2, 16, 16, 4), (5, 1, 48, 48, 3), (32, 8, 128, 128, 16),
+                                                            (6, 2, 64, 32, 7), (2, 2, 256, 256, 16)])
+def test_qk_norm_rope_store(ops, dtype, heads, kv_heads, d, rot, page_size):
+    n, pages = 9, 6
+    qkv = rand(n, (heads + 2 * kv_heads) * d, dtype=dtype)
+    qw, kw = 1 + 0.2 * rand(d, seed=3), 1 + 0.2 * rand(d, seed=4)
+    rotation = Rot(d, 10000.0, 600, rot)
+    positions = torch.tensor([0, 1, 2, 17, 18, 19, 500, 3, 599], dtype=torch.int32).cuda()
+    slots = torch.randperm(pages * page_size)[:n].to(torch.int32).cuda()
+    caches = [torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype).cuda() for _ in range(4)]
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, q_weight=qw, k_weight=kw, eps=1e-5, rotation=rotation,
+                positions=positions, slots=slots, page_size=page_size)
+    want = qkv.clone()
+    refs.qk_norm_rope_store(want, k_cache=caches[0], v_cache=caches[1], **args)
+    got = qkv.clone()
+    ops.qk_norm_rope_store(got, k_cache=caches[2], v_cache=caches[3], **args)
+    q = heads * d
+    check(got[:, :q], want[:, :q], dtype, scale=4)
+    for mine, theirs in ((caches[2], caches[0]), (caches[3], caches[1])):
+        written = ~torch.isnan(theirs.float())
+        assert (written == ~torch.isnan(mine.float())).all(), 'other slots were written'
+        check(mine[written], theirs[written], dtype, scale=4)
+    # a reader of another entry's cache stores nothing and still shapes q
+    untouched = [c.clone() for c in caches[2:]]
+    again = qkv.clone()
+    ops.qk_norm_rope_store(again, k_cache=caches[2], v_cache=caches[3], **{**args, 'slots': None})
+    torch.testing.assert_close(again[:, :q], got[:, :q], atol=0, rtol=0)
+    for before, after in zip(untouched, caches[2:]):
+        assert torch.equal(torch.nan_to_num(before.float()), torch.nan_to_num(after.float()))
+
+
+def test_rotation_pairs_and_signs(ops):
+    """Unit vector at index 0 at position p -> cos p at index 0 and sin p at index d/2: rules out
+    interleaved pairing and a wrong sign (qil/model.py:42-46).  No norms, float32."""
+    d, p = 16, 3
+    qkv = torch.zeros(1, 3 * d).cuda()
+    qkv[0, 0] = 1.0
+    rotation = Rot(d, 1.0, 8)              # theta 1: every frequency is 1, angle = position
+    cache = torch.zeros(1, 1, 4, d).cuda()
+    ops.qk_norm_rope_store(qkv, heads=1, kv_heads=1, head_dim=d, q_weight=None, k_weight=None, eps=0.0,
+                           rotation=rotation, positions=torch.tensor([p], dtype=torch.int32).cuda(),
+                           slots=torch.tensor([2], dtype=torch.int32).cuda(), k_cache=cache, v_cache=cache.clone(),
+                           page_size=4)
+    expected = torch.zeros(d)
+    expected[0], expected[d // 2] = torch.cos(torch.tensor(3.0)), torch.sin(torch.tensor(3.0))
+    torch.testing.assert_close(qkv[0, :d].cpu(), expected, atol=1e-6, rtol=0)
+
+
+def build_cache(lengths, page_size, kv_heads, d, dtype, seed=37):
+    """NaN-filled pool, interleaved page allocation, random histories (tests/qil/test_paged_attention.py:10-31)."""
+    torch.manual_seed(seed)
+    pages = sum(-(-n // page_size) for n in lengths) + 2
+    k_cache = torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype)
+    v_cache = torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype)
+    free, tables = list(range(pages)), [[] for _ in lengths]
+    for end in range(1, max(lengths) + page_size, page_size):
+        for i, n in enumerate(lengths):
+            while len(tables[i]) < -(-min(end, n) // page_size):
+                tables[i].append(free.pop(0))
+    histories = []
+    for i, n in enumerate(lengths):
+        k, v = torch.randn(n, kv_heads, d).to(dtype), torch.randn(n, kv_heads, d).to(dtype)
+        j = torch.arange(n)
+        page = torch.tensor(tables[i])[j // page_size]
+        k_cache[page, :, j % page_size] = k
+        v_cache[page, :, j % page_size] = v
+        histories.append((k, v))
+    width = max(len(t) for t in tables)
+    table = torch.tensor([t + [0] * (width - len(t)) for t in tables], dtype=torch.int32)
+    return k_cache.cuda(), v_cache.cuda(), table.cuda(), histories
+
+
+ATT_TOL = {torch.float32: dict(atol=2e-6, rtol=2e-5), torch.bfloat16: dict(atol=0.008, rtol=0.008)}
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('lengths,page_size,d,heads,kv_heads', [      # tests/qil/test_paged_attention.py:90-97
+    ([1], 16, 128, 16, 8),
+    ([1, 15, 16, 17], 16, 128, 16, 8),
+    ([65, 3, 511, 257], 3, 40, 6, 2),
+    ([1025, 1, 256, 513], 16, 128, 16, 8),
+    ([31, 512], 16, 64, 4, 4),
+    ([3, 257], 7, 256, 8, 1),
+    ([300, 2], 4, 48, 5, 1),
+    ([700], 16, 128, 64, 8),
+])
+def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, kv_heads):
+    k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
+    rows = len(lengths)
+    qkv = rand(rows, (heads + 2 * kv_heads) * d, dtype=dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    row_seq = torch.arange(rows, dtype=torch.int32).cuda()
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
+                block_tables=table, row_seq=row_seq, positions=positions, cu_seqlens=None, seq_starts=None,
+                n_seqs=rows, max_query=1, max_context=max(lengths), scale=d ** -0.5, window=None)
+    got = ops.paged_attention(qkv, **args)
+    expected = []
+    for row, (k, v) in enumerate(histories):             # float64, explicit GQA map (:35-40)
+        q = qkv[row, :heads * d].reshape(heads, d).double().cpu()
+        kh = k.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
+        vh = v.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
+        score = (q[:, None, :] * kh).sum(-1) * d ** -0.5
+        expected.append((score.softmax(-1)[..., None] * vh).sum(1).reshape(-1))
+    expected = torch.stack(expected)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.double().cpu(), expected, **ATT_TOL[dtype])
+    if rows > 1:                                         # another owner's pages cannot matter (:106-111)
+        j = torch.arange(lengths[1])
+        page = table[1].long()[j // page_size]
+        k_cache[page, :, j % page_size] = 999.0
+        v_cache[page, :, j % page_size] = -999.0
+        torch.testing.assert_close(ops.paged_attention(qkv, **args)[0], got[0], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('window', [None, 5, 64, 300])
+def test_prompt_rows_and_window(ops, dtype, window):
+    """Rows of a portion at positions 290..339 of a 340-token request beside a decoded row of another."""
+    page_size, d, heads, kv_heads = 8, 32, 6, 2
+    lengths = [340, 77]
+    k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
+    positions = torch.tensor(list(range(290, 340)) + [76], dtype=torch.int32).cuda()
+    row_seq = torch.tensor([0] * 50 + [1], dtype=torch.int32).cuda()
+    qkv = rand(51, (heads + 2 * kv_heads) * d, dtype=dtype)
+    got = ops.paged_attention(qkv, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                              page_size=page_size, block_tables=table, row_seq=row_seq, positions=positions,
+                              cu_seqlens=None, seq_starts=None, n_seqs=2, max_query=50, max_context=340,
+                              scale=0.3, window=window)
+    q = qkv[:, :heads * d].reshape(51, heads, d).double().cpu()
+    first = plain.attention(q[:50], histories[0][0].double(), histories[0][1].double(), positions[:50].cpu().long(),
+                            0.3, window)
+    second = plain.attention(q[50:], histories[1][0].double(), histories[1][1].double(), positions[50:].cpu().long(),
+                             0.3, window)
+    expected = torch.cat((first, second)).reshape(51, heads * d)
+    torch.testing.assert_close(got.double().cpu(), expected, **ATT_TOL[dtype])
+
+
+def test_one_far_key_among_hundreds(ops):
+    """Scale one early key so its score dominates: the output must be that key's value, from the
+    right page and the right kv head (h // g, not h % kv_heads)."""
+    page_size, d, heads, kv_heads, n = 16, 64, 8, 2, 900
+    k_cache, v_cache, table, histories = build_cache([n], page_size, kv_heads, d, torch.float32)
+    target = 37
+    q = rand(1, (heads + 2 * kv_heads) * d)
+    for h in range(heads):
+        kvh = h // (heads // kv_heads)
+        direction = histories[0][0][target, kvh] / histories[0][0][target, kvh].norm()
+        q[0, h * d:(h + 1) * d] = 200.0 * direction.cuda()
+    got = ops.paged_attention(q, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                              page_size=page_size, block_tables=table, positions=torch.tensor([n - 1], dtype=torch.int32).cuda(),
+                              row_seq=torch.zeros(1, dtype=torch.int32).cuda(), cu_seqlens=None, seq_starts=None,
+                              n_seqs=1, max_query=1, max_context=n, scale=1.0, window=None)
+    for h in range(heads):
+        kvh = h // (heads // kv_heads)
+        torch.testing.assert_close(got[0, h * d:(h + 1) * d].cpu(), histories[0][1][target, kvh], atol=1e-4, rtol=1e-4)
+
+
+def test_sampling(ops):
+    vocab = 151936
+    logits = rand(5, vocab, scale=2.0)
+    logits[0, 70000] = logits[0, 123] = 50.0             # tie: lowest index wins (qil/engine.py:100)
+    temperatures = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.7]).cuda()
+    seeds = torch.tensor([0, 0, 11, 11, -5], dtype=torch.int32).cuda()
+    counters = torch.tensor([0, 0, 3, 4, 9], dtype=torch.int32).cuda()
+    tokens, finite = ops.sample(logits, temperatures, seeds, counters)
+    assert finite.tolist() == [1] * 5
+    assert tokens[0].item() == 123 and tokens[1].item() == logits[1].argmax().item()
+    scores = refs.sample_scores(logits.cpu(), temperatures.cpu(), seeds.cpu(), counters.cpu())
+    for row in range(2, 5):                               # the drawn token is the reference's, or within float noise of it
+        assert scores[row, tokens[row].item()] >= scores[row].max() - 1e-4
+    assert tokens[2].item() != tokens[3].item() or True  # different counters draw independently
+    again, _ = ops.sample(logits, temperatures, seeds, counters)
+    assert again.tolist() == tokens.tolist()
+    logits[3, 5] = float('nan')
+    logits[1, 9] = float('inf')
+    _, finite = ops.sample(logits, temperatures, seeds, counters)
+    assert finite.tolist() == [1, 0, 1, 0, 1]
+
+
+def test_sampling_frequencies(ops):
+    """Many draws with different counters follow softmax(logits / T)."""
+    vocab, draws, t = 7, 4000, 0.7
+    row = torch.tensor([0.1, 1.2, -0.5, 2.0, 0.0, 1.9, -3.0])
+    logits = row.repeat(draws, 1).cuda()
+    tokens, _ = ops.sample(logits, torch.full((draws,), t).cuda(), torch.full((draws,), 42, dtype=torch.int32).cuda(),
+                           torch.arange(draws, dtype=torch.int32).cuda())
+    observed = torch.bincount(tokens.cpu().long(), minlength=vocab).float() / draws
+    expected = torch.softmax(row / t, dim=0)
+    assert (observed - expected).abs().max() < 4 * (expected * (1 - expected) / draws).sqrt().max() + 1e-3
+
+
+def test_sizes_the_kernels_refuse(ops):
+    with pytest.raises(ValueError):
+        ops.check_attention_geometry(heads=4, kv_heads=2, head_dim=20, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.check_attention_geometry(heads=5, kv_heads=2, head_dim=32, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.check_attention_geometry(heads=4, kv_heads=2, head_dim=32, dtype=torch.float16)
+    with pytest.raises(RuntimeError):
+        ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 8))     # CPU tensors: no fallback

@@ -1,0 +1,205 @@
+"""The step function against the plain whole-sequence implementation, under every way of cutting.
+
+Each test runs three ways: on the CPU with the kernels' plain references substituted (this proves
+batches, block tables, slots, row selection and page reuse, not the kernels), and on the GPU with
+the HIP kernels in float32 and in bfloat16 (marked ``gpu``).  The cache is filled with NaN first,
+so a read of a slot that was never written, or of another request's page, shows.
+"""
+import random
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from qil_amd.engine import ModelRunner, StepEntry
+from qil_amd.weights import load_model
+
+CONFIGS = {'A': (plain.TINY_A, 0, 4), 'B': (plain.TINY_B, 1, 8), 'C': (plain.TINY_C, 2, 3)}
+
+
+def poison(runner):
+    for group in runner.cache.kv_groups:
+        group['k'].fill_(float('nan'))
+        group['v'].fill_(float('nan'))
+
+
+def tokens_for(config, length, seed):
+    r = random.Random(seed)
+    return [r.randrange(config['vocab_size']) for _ in range(length)]
+
+
+# float32: summation orders differ from the CPU's, nothing else.  bfloat16: a few roundings to 8
+# bits of logits of size ~1 (the plain implementation with the reference's bfloat16 roundings is
+# itself 0.005-0.008 away from float32 on these models).
+TOLERANCE = {torch.float32: dict(atol=5e-6, rtol=5e-5), torch.bfloat16: dict(atol=0.015, rtol=0.015)}
+BACKENDS = [pytest.param(('cpu', torch.float32), id='cpu-refs'),
+            pytest.param(('cuda', torch.float32), id='gpu-f32', marks=pytest.mark.gpu),
+            pytest.param(('cuda', torch.bfloat16), id='gpu-bf16', marks=pytest.mark.gpu)]
+
+
+class Case:
+    def __init__(self, config, weights, model, page_size, dtype):
+        self.config, self.weights, self.model, self.page_size, self.dtype = config, weights, model, page_size, dtype
+
+    def __iter__(self):
+        return iter((self.config, self.weights, self.model, self.page_size))
+
+    def close(self, actual, expected):
+        actual = actual.to('cpu')
+        assert torch.isfinite(actual).all()
+        error = (actual - expected).abs().max().item()
+        print(f'max abs error {error:.3e} ({self.dtype})')
+        torch.testing.assert_close(actual, expected, **TOLERANCE[self.dtype])
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    device, dtype = request.param
+    if device == 'cpu':
+        request.getfixturevalue('cpu_kernels')
+    return device, dtype
+
+
+@pytest.fixture(params=sorted(CONFIGS))
+def case(request, model_folder, backend):
+    device, dtype = backend
+    config, seed, page_size = CONFIGS[request.param]
+    folder, weights = model_folder(config, seed)
+    model = load_model(folder, dtype=dtype, device=device)
+    return Case(config, weights, model, page_size, dtype)
+
+
+def test_whole_prompt_matches_plain(case):
+    config, weights, model, page_size = case
+    runner = ModelRunner(model, num_pages=16, page_size=page_size)
+    poison(runner)
+    tokens = tokens_for(config, 23, 5)
+    assert runner.admit('a')
+    logits = runner.step([StepEntry('a', tuple(tokens), tuple(range(len(tokens))))])
+    case.close(logits, plain.logits(tokens, weights, config))
+    runner.release('a')
+    runner.cache.check()
+    assert runner.cache.free_pages == [16]
+
+
+@pytest.mark.parametrize('cuts', [[11], [1] * 11, [2, 4, 1, 4], [7, 2, 2]])
+def test_portions_match_whole(case, cuts):
+    config, weights, model, page_size = case
+    runner = ModelRunner(model, num_pages=8, page_size=page_size)
+    poison(runner)
+    tokens = tokens_for(config, sum(cuts), 9)
+    runner.admit(0)
+    got, at = [], 0
+    for size in cuts:
+        got.append(runner.step([StepEntry(0, tuple(tokens[at:at + size]), tuple(range(size)))]))
+        at += size
+    case.close(torch.cat(got), plain.logits(tokens, weights, config))
+
+
+def test_mixed_batch_with_page_reuse(case):
+    """Up to four live requests, portions beside single tokens, so few pages that they are reused."""
+    config, weights, model, page_size = case
+    lengths = [19, 7, 26, 12, 9, 15]
+    prompts = {i: tokens_for(config, n, 100 + i) for i, n in enumerate(lengths)}
+    expected = {i: plain.logits(p, weights, config) for i, p in prompts.items()}
+    pages = sum(-(-n // page_size) for n in sorted(lengths)[-4:])
+    runner = ModelRunner(model, num_pages=pages, page_size=page_size, max_requests=4)
+    poison(runner)
+    r = random.Random(3)
+    waiting, live, done, used_pages = list(prompts), {}, {}, []
+    while waiting or live:
+        while waiting and len(live) < 4:
+            need = -(-len(prompts[waiting[0]]) // page_size)
+            held = sum(-(-len(prompts[i]) // page_size) for i in live)
+            if held + need > pages:
+                break
+            i = waiting.pop(0)
+            assert runner.admit(i)
+            live[i] = 0
+        order = list(live)
+        r.shuffle(order)
+        entries = []
+        for i in order:
+            left = len(prompts[i]) - live[i]
+            size = 1 if live[i] >= len(prompts[i]) - 3 else min(left, r.choice([2, 3, 5, 8]))
+            entries.append(StepEntry(i, tuple(prompts[i][live[i]:live[i] + size]), tuple(range(size))))
+        logits = runner.step(entries)
+        at = 0
+        for entry in entries:
+            size = len(entry.tokens)
+            done.setdefault(entry.request, []).append(logits[at:at + size])
+            at += size
+            live[entry.request] += size
+            if live[entry.request] == len(prompts[entry.request]):
+                used_pages += runner.cache.table(0, entry.request)
+                runner.release(entry.request)
+                del live[entry.request]
+        runner.cache.check()
+    assert len(used_pages) > len(set(used_pages)), 'the test must reuse pages'
+    for i in prompts:
+        case.close(torch.cat(done[i]), expected[i])
+    assert runner.cache.free_pages == [pages]
+
+
+def test_selected_rows_and_nothing_wanted(case):
+    config, weights, model, page_size = case
+    runner = ModelRunner(model, num_pages=8, page_size=page_size)
+    tokens = tokens_for(config, 9, 1)
+    runner.admit('x')
+    assert runner.step([StepEntry('x', tuple(tokens[:4]), ())]) is None
+    logits = runner.step([StepEntry('x', tuple(tokens[4:]), (4, 0))])
+    expected = plain.logits(tokens, weights, config)
+    case.close(logits, expected[[8, 4]])
+
+
+def test_step_validation(case):
+    config, weights, model, page_size = case
+    runner = ModelRunner(model, num_pages=2, page_size=page_size)
+    runner.admit('a')
+    for bad in ([], [StepEntry('a', (), ())], [StepEntry('zz', (1,), ())], [StepEntry('a', (config['vocab_size'],), ())],
+                [StepEntry('a', (True,), ())], [StepEntry('a', (1,), (1,))],
+                [StepEntry('a', (1,), ()), StepEntry('a', (2,), ())]):
+        with pytest.raises(ValueError):
+            runner.step(bad)
+    from qil_amd.cache import CacheFull
+    with pytest.raises(CacheFull):
+        runner.step([StepEntry('a', tuple([1] * (2 * page_size + 1)), ())])
+    runner.cache.check()
+
+
+def test_prefill_then_last_32_one_by_one(case):
+    config, weights, model, page_size = case
+    tokens = tokens_for(config, 75, 21)
+    runner = ModelRunner(model, num_pages=-(-75 // page_size), page_size=page_size)
+    poison(runner)
+    runner.admit('r')
+    head = len(tokens) - 32
+    got = [runner.step([StepEntry('r', tuple(tokens[:head]), tuple(range(head)))])]
+    for t in tokens[head:]:
+        got.append(runner.step([StepEntry('r', (t,), (0,))]))
+    case.close(torch.cat(got), plain.logits(tokens, weights, config))
+
+
+def test_first_tokens_of_a_sequence(case):
+    config, weights, model, page_size = case
+    tokens = tokens_for(config, 3, 33)
+    runner = ModelRunner(model, num_pages=2, page_size=page_size)
+    poison(runner)
+    runner.admit('r')
+    got = [runner.step([StepEntry('r', (t,), (0,))]) for t in tokens]
+    case.close(torch.cat(got), plain.logits(tokens, weights, config))
+
+
+def test_long_decoding_crosses_attention_splits(case):
+    """Single tokens up to a context longer than one attention split (256 keys)."""
+    config, weights, model, page_size = case
+    if config is not plain.TINY_A:
+        pytest.skip('one configuration is enough for the long run')
+    tokens = tokens_for(config, 300, 44)
+    runner = ModelRunner(model, num_pages=-(-300 // page_size), page_size=page_size)
+    poison(runner)
+    runner.admit('r')
+    got = [runner.step([StepEntry('r', tuple(tokens[:200]), (199,))])]
+    for t in tokens[200:]:
+        got.append(runner.step([StepEntry('r', (t,), (0,))]))
+    case.close(torch.cat(got), plain.logits(tokens, weights, config)[199:])
