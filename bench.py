@@ -1,0 +1,154 @@
+"""Decode and prefill throughput of the engine at Qwen3-8B sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16]
+
+Random weights, seeded uniform-random token ids.  A step is one decode step of the
+serving loop (scheduler plan, one batched model step, greedy sampling, events) with
+every request decoding at a 2,048-token history.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import statistics
+import sys
+import time
+
+HBM_GBPS = 8000.0                                   # MI355X published peaks
+PEAK_TFLOPS = {'bfloat16': 2500.0, 'float32': 157.3}
+
+SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
+             num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096,
+             rms_norm_eps=1e-6, rope_theta=1000000.0, attention_bias=False, tie_word_embeddings=False,
+             model_type='qwen3', architectures=['Qwen3ForCausalLM'], hidden_act='silu', eos_token_id=None)
+
+
+def matrix_params_per_layer(c):
+    qkv = (c['num_attention_heads'] + 2 * c['num_key_value_heads']) * c['head_dim'] * c['hidden_size']
+    out = c['num_attention_heads'] * c['head_dim'] * c['hidden_size']
+    return qkv + out + 3 * c['hidden_size'] * c['intermediate_size']
+
+
+def decode_bytes(c, element, contexts):
+    """Every weight the step uses once, and the cache of the live requests."""
+    layers = c['num_hidden_layers']
+    weights = layers * (matrix_params_per_layer(c) * element + (2 * c['hidden_size'] + 2 * c['head_dim']) * 4)
+    weights += c['vocab_size'] * c['hidden_size'] * element + c['hidden_size'] * 4
+    kv = sum(contexts) * layers * 2 * c['num_key_value_heads'] * c['head_dim'] * element
+    return weights + kv + len(contexts) * c['hidden_size'] * element          # + the embedding rows
+
+
+def prefill_flops(c, tokens):
+    layers = c['num_hidden_layers']
+    linear = 2 * tokens * layers * matrix_params_per_layer(c) + 2 * c['vocab_size'] * c['hidden_size']
+    attention = layers * 4 * c['num_attention_heads'] * c['head_dim'] * tokens * (tokens + 1) // 2
+    return linear + attention
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument('--gpus', type=int, default=1)
+    parser.add_argument('--steps', type=int, default=64)
+    parser.add_argument('--warmup', type=int, default=8)
+    parser.add_argument('--layers', type=int, default=SIZES['num_hidden_layers'])
+    parser.add_argument('--batch', type=int, default=8)
+    parser.add_argument('--history', type=int, default=2048)
+    parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
+    parser.add_argument('--points', default='1,64', help='other decode batch sizes to report, comma separated')
+    parser.add_argument('--prefill-tokens', type=int, default=2048)
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py measures one GPU: this engine runs on a single MI355X (asked for {args.gpus})')
+        return 2
+
+    import torch
+    from qil_amd import Engine, Qwen3
+    from qil_amd.engine import ModelRunner, StepEntry
+
+    config = dict(SIZES, num_hidden_layers=args.layers)
+    dtype = getattr(torch, args.dtype)
+    element = 2 if args.dtype == 'bfloat16' else 4
+    model = Qwen3.from_config(config, seed=0, dtype=dtype, device='cuda:0', on_device=True)
+    generator = torch.Generator().manual_seed(1234)
+    page_size = 16
+
+    def prompt(length):
+        return torch.randint(0, config['vocab_size'], (length,), generator=generator).tolist()
+
+    def decode_run(batch):
+        """(seconds per step, contexts at the middle of the timed steps) of `batch` requests decoding together."""
+        new_tokens = args.warmup + args.steps + 2
+        pages = batch * (-(-(args.history + new_tokens) // page_size) + 1)
+        engine = Engine(model, num_pages=pages, page_size=page_size, token_budget=args.history + batch,
+                        prefill_chunk=args.history, max_active=batch)
+        ids = [engine.submit(prompt(args.history), max_new_tokens=new_tokens + batch, ignore_eos=True)
+               for _ in range(batch)]
+        requests = engine.scheduler.requests
+        while any(requests[i].computed < args.history for i in ids):      # untimed: histories into the cache
+            engine.step()
+        for _ in range(args.warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        produced = 0
+        for _ in range(args.steps):
+            produced += len(engine.step())
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        assert produced == batch * args.steps, 'a decode step must produce one token per request'
+        contexts = [requests[i].computed - args.steps // 2 for i in ids]
+        engine.close()
+        engine.cache.check()
+        assert engine.cache.free_pages == [pages], 'pages leaked'
+        del engine
+        torch.cuda.empty_cache()
+        return elapsed / args.steps, contexts
+
+    def prefill_run(tokens):
+        runner = ModelRunner(model, num_pages=-(-tokens // page_size) + 1, page_size=page_size, max_requests=1)
+        times = []
+        for attempt in range(4):
+            ids = tuple(prompt(tokens))
+            runner.admit(attempt)
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            logits = runner.step([StepEntry(attempt, ids, (tokens - 1,))])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - started)
+            assert torch.isfinite(logits).all()
+            runner.release(attempt)
+        return statistics.median(times[1:])
+
+    step_s, contexts = decode_run(args.batch)
+    points = {}
+    for batch in [int(b) for b in args.points.split(',') if b]:
+        seconds, _ = decode_run(batch)
+        points[f'decode_b{batch}'] = round(batch / seconds, 1)
+    prefill_s = prefill_run(args.prefill_tokens)
+
+    value = args.batch / step_s
+    bytes_read = decode_bytes(config, element, contexts)
+    achieved = bytes_read / step_s / 1e9
+    flops = prefill_flops(config, args.prefill_tokens)
+    line = {
+        'metric': 'decode tok/s at batch 8 (Qwen3-8B sizes, 2048-token histories)', 'value': round(value, 1),
+        'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(step_s * 1e3, 4), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16' if args.dtype == 'bfloat16' else 'fp32', 'data': 'synthetic',
+        'config': {'model': 'Qwen3-8B sizes, random weights', 'layers': args.layers,
+                   'layers_of_model': SIZES['num_hidden_layers'], 'hidden': config['hidden_size'],
+                   'heads': config['num_attention_heads'], 'kv_heads': config['num_key_value_heads'],
+                   'head_dim': config['head_dim'], 'intermediate': config['intermediate_size'],
+                   'vocab': config['vocab_size'], 'global_batch': args.batch, 'seq_len': args.history,
+                   'context': config['max_position_embeddings'], 'page_size': page_size,
+                   'prefill_tokens': args.prefill_tokens, 'parallelism': 'single GPU'},
+        'prefill': {'value': round(args.prefill_tokens / prefill_s, 1), 'tokens': args.prefill_tokens,
+                    'ms': round(prefill_s * 1e3, 3), 'frac': round(flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+        'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_GBPS, 'unit': 'GB/s',
+                     'frac': round(achieved / HBM_GBPS, 4)},
+        'points': points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == '__main__':
+    sys.exit(main())

@@ -29,11 +29,13 @@ __global__ void __launch_bounds__(ATT_THREADS)
 attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
                          const T* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                          const int* __restrict__ row_seq, const int* __restrict__ positions,
-                         float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l,
+                         const int* __restrict__ row_index, float* __restrict__ part_acc,
+                         float* __restrict__ part_m, float* __restrict__ part_l,
                          T* __restrict__ out, int heads, int kv_heads, int d, int page_size, int window,
                          float scale, int P, int parts, int tg_log2) {
   extern __shared__ float lds[];
-  const int row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
+  const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;   // slot_row indexes the workspace
+  const int row = row_index ? row_index[slot_row] : slot_row;             // row of the step's batch
   const int g = heads / kv_heads;
   const int ctx = positions[row] + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
@@ -43,7 +45,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
 
   const int TG = 1 << tg_log2, TPW = QIL_WAVE >> tg_log2;
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
-  const int sub = lane & (TG - 1), slot = lane >> tg_log2;
+  const int sub = lane & (TG - 1), slot = lane >> tg_log2;   // slot: which token of the wave's group
   const int e0 = sub * 8;
   const bool live = e0 < d;                       // lanes past d (padding of TG to a power of two) idle
   const int* table = block_tables + (size_t)row_seq[row] * table_stride;
@@ -152,7 +154,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
       if (parts == 1) {
         st(out + ((size_t)row * heads + head) * d + e, total / l);
       } else {
-        const size_t cell = ((size_t)row * heads + head) * parts + part;
+        const size_t cell = ((size_t)slot_row * heads + head) * parts + part;
         part_acc[cell * d + e] = total;
         if (e == 0) { part_m[cell] = m; part_l[cell] = l; }
       }
@@ -164,12 +166,14 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
 template <typename T>
 __global__ void attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
                                        const float* __restrict__ part_l, const int* __restrict__ positions,
-                                       T* __restrict__ out, int heads, int d, int window, int P, int parts) {
-  const int row = blockIdx.x, head = blockIdx.y;
+                                       const int* __restrict__ row_index, T* __restrict__ out, int heads, int d,
+                                       int window, int P, int parts) {
+  const int slot_row = blockIdx.x, head = blockIdx.y;
+  const int row = row_index ? row_index[slot_row] : slot_row;
   const int ctx = positions[row] + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
   const int first = lo / P, last = (ctx - 1) / P;
-  const size_t cell0 = ((size_t)row * heads + head) * parts;
+  const size_t cell0 = ((size_t)slot_row * heads + head) * parts;
   float m = -INFINITY;
   for (int p = first; p <= last; ++p) m = fmaxf(m, part_m[cell0 + p]);
   float denom = 0.f;
@@ -192,7 +196,8 @@ static size_t rows_lds_floats(int gt, int P, int d) { return (size_t)gt * P + 16
 
 template <typename T>
 static int launch_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
-                       int table_stride, const int* row_seq, const int* positions, float* part_acc, float* part_m,
+                       int table_stride, const int* row_seq, const int* positions, const int* row_index,
+                       float* part_acc, float* part_m,
                        float* part_l, void* out, int rows, int heads, int kv_heads, int d, int page_size, int window,
                        float scale, int P, int parts, hipStream_t s) {
   const int g = heads / kv_heads;
@@ -203,7 +208,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
 #define QIL_ROWS_CASE(GT)                                                                                          \
   hipLaunchKernelGGL((attn_rows_partial_kernel<T, GT>), grid, dim3(ATT_THREADS), lds, s, (const T*)q, q_stride,    \
                      (const T*)k_cache, (const T*)v_cache, block_tables, table_stride, row_seq, positions,         \
-                     part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, P, parts,    \
+                     row_index, part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, P, parts,    \
                      tg_log2)
   switch (gt) {
     case 1: QIL_ROWS_CASE(1); break;
@@ -215,7 +220,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
   int status = (int)hipGetLastError();
   if (status || parts == 1) return status;
   hipLaunchKernelGGL(attn_rows_merge_kernel<T>, dim3(rows, heads), dim3(d >= 128 ? 128 : 64), 0, s, part_acc, part_m,
-                     part_l, positions, (T*)out, heads, d, window, P, parts);
+                     part_l, positions, row_index, (T*)out, heads, d, window, P, parts);
   return (int)hipGetLastError();
 }
 
@@ -226,11 +231,13 @@ size_t qil_attn_rows_workspace(int rows, int heads, int d, int parts) {
   return parts <= 1 ? 0 : (size_t)rows * heads * parts * (d + 2) * sizeof(float);
 }
 
-// q: rows of stride q_stride elements, head h at offset h * d.  out: [rows, heads * d].
+// q: rows of stride q_stride elements, head h at offset h * d.  out: [all rows, heads * d].
+// row_index: null (the kernel's rows are the batch's rows 0 .. rows-1) or the batch rows to serve.
 // workspace: qil_attn_rows_workspace bytes.  P: keys per part, parts = ceil(max context / P).
 // Requires d % 8 == 0, d <= 256, P <= 1024.  Returns -1 on a size it does not take.
 int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
-                  int table_stride, const int* row_seq, const int* positions, void* workspace, void* out, int rows,
+                  int table_stride, const int* row_seq, const int* positions, const int* row_index, void* workspace,
+                  void* out, int rows,
                   int heads, int kv_heads, int d, int page_size, int window, float scale, int P, int parts, int dtype,
                   hipStream_t s) {
   if (rows == 0) return 0;
@@ -243,10 +250,10 @@ int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* 
   float* m = acc ? acc + (size_t)rows * heads * parts * d : nullptr;
   float* l = m ? m + (size_t)rows * heads * parts : nullptr;
   if (dtype == QIL_F32)
-    return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, acc, m, l,
-                              out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
-  return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, acc, m, l,
-                             out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+    return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
+                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+  return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
+                             acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
 }
 
 }  // extern "C"

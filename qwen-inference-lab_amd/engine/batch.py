@@ -29,6 +29,7 @@ class StepContext:
     seq_starts: torch.Tensor       # [S] position of each sequence's first row (cached length before the step)
     seq_slots: torch.Tensor        # [S] state slot of each sequence's request
     logit_rows: torch.Tensor       # [M] rows whose logits are wanted
+    single_rows: torch.Tensor      # rows that are alone in their sequence; None if every row is (max_query == 1)
     max_query: int                 # most rows of one sequence
     max_context: int               # largest position + 1
     host_cu_seqlens: list = field(default_factory=list)

@@ -50,7 +50,8 @@ class Engine:
         if not plan:
             return []
         requests = self.scheduler.requests
-        ready = [w.start + len(w.tokens) == len(requests[w.request_id].input_tokens) for w in plan]
+        ready = [w.start + len(w.tokens) == len(requests[w.request_id].prompt) + len(requests[w.request_id].output)
+                 for w in plan]
         try:
             entries = [StepEntry(w.request_id, w.tokens, (len(w.tokens) - 1,) if r else ())
                        for w, r in zip(plan, ready)]

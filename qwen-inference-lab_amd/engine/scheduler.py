@@ -84,12 +84,18 @@ class Scheduler:
                 break
             request_id = self.active.popleft()
             request = self.requests[request_id]
-            inputs = request.input_tokens
-            chunk = self.prefill_chunk if request.computed < len(request.prompt) else 1
-            count = min(chunk, remaining, len(inputs) - request.computed)
+            at, prompt_length = request.computed, len(request.prompt)
+            chunk = self.prefill_chunk if at < prompt_length else 1
+            count = min(chunk, remaining, prompt_length + len(request.output) - at)
             if count <= 0:
                 raise RuntimeError('active request has no input to compute')
-            work.append(Work(request_id, request.computed, tuple(inputs[request.computed:request.computed + count])))
+            if at + count <= prompt_length:           # slices, not prompt + output: that copy grows with the context
+                tokens = request.prompt[at:at + count]
+            elif at >= prompt_length:
+                tokens = request.output[at - prompt_length:at - prompt_length + count]
+            else:
+                tokens = request.prompt[at:] + request.output[:at + count - prompt_length]
+            work.append(Work(request_id, at, tuple(tokens)))
             remaining -= count
             self.active.append(request_id)
         if not work and self.waiting:

@@ -82,7 +82,8 @@ class ModelRunner:
         slots = [cache.slots[e.request] for e in entries]
         max_context = int(max(st + c for st, c in zip(starts, counts)))
 
-        pieces = [tokens, positions, row_seq, cu, np.asarray(starts), np.asarray(slots), logit_rows]
+        single = cu[:-1][np.asarray(counts) == 1] if max(counts) > 1 else np.zeros(0, dtype=np.int64)
+        pieces = [tokens, positions, row_seq, cu, np.asarray(starts), np.asarray(slots), logit_rows, single]
         group_tables = []
         for index, group in enumerate(cache.kv_groups):
             tables = [cache.table(index, e.request) for e in entries]
@@ -104,6 +105,7 @@ class ModelRunner:
         ctx = StepContext(
             n_tokens=n, n_seqs=s, n_logit_rows=len(logit_rows), token_ids=part(0), positions=part(1),
             row_seq=part(2), cu_seqlens=part(3), seq_starts=part(4), seq_slots=part(5), logit_rows=part(6),
+            single_rows=part(7) if max(counts) > 1 else None,
             max_query=max(counts), max_context=max_context, host_cu_seqlens=cu.tolist(), host_starts=starts,
             host_slots=slots, requests=[e.request for e in entries])
         for view in self.views:

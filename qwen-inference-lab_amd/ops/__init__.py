@@ -183,12 +183,16 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 
 def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
-                    cu_seqlens, seq_starts, n_seqs, max_query, max_context, scale, window):
+                    cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window):
     """Attention of every row of the step over its request's cached keys.
 
     q is read from the leading ``heads * head_dim`` columns of ``qkv`` [N, (heads + 2 kv_heads) d].
     Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
     j <= positions[n] and, with a window, j > positions[n] - window.  -> T [N, heads * head_dim].
+
+    Sequences with two or more rows (``cu_seqlens``, ``seq_starts``) go to the matrix-core tile
+    kernel; rows alone in their sequence (``single_rows``: their indices, or None when every row is
+    alone, i.e. ``max_query == 1``) go to the split-context row kernel.
     """
     n = qkv.shape[0]
     check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=head_dim, dtype=qkv.dtype)
@@ -203,15 +207,31 @@ def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_si
     if block_tables.ndim != 2 or block_tables.shape[1] * page_size < max_context:
         raise ValueError('block_tables are too narrow for the longest context')
     lib = library.load()
-    part = ATTENTION_PART
-    parts = max(1, -(-max_context // part))
     out = torch.empty((n, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    nbytes = lib.qil_attn_rows_workspace(n, heads, head_dim, parts)
-    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
-    _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
-                             block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(workspace), _ptr(out), n,
-                             heads, kv_heads, head_dim, page_size, int(window or 0), float(scale), part, parts,
-                             _code(qkv.dtype), _stream()), 'attn_rows')
+    if max_query > 1:
+        _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+        _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+        if block_tables.shape[0] != n_seqs:
+            raise ValueError('one block table row per sequence')
+        _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                 block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
+                                 max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
+                                 _code(qkv.dtype), _stream()), 'attn_tile')
+        if single_rows is None:
+            raise ValueError('single_rows must list the rows that are alone when some sequence has several')
+        _require(single_rows, 'single_rows', torch.int32)
+        rows = single_rows.shape[0]
+    else:
+        single_rows, rows = None, n
+    if rows:
+        part = ATTENTION_PART
+        parts = max(1, -(-max_context // part))
+        nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
+        workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
+        _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                 block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
+                                 _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
+                                 int(window or 0), float(scale), part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
     return out
 
 

@@ -144,10 +144,11 @@ def _declare(lib):
     lib.qil_qk_norm_rope_store.argtypes = [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, p]
     lib.qil_attn_rows_workspace.argtypes = [i, i, i, i]
     lib.qil_attn_rows_workspace.restype = z
-    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, p]
     lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_sample.argtypes = [p, p, p, p, p, p, i, i, p]
     for name in ('qil_embed', 'qil_add_rmsnorm', 'qil_silu_mul', 'qil_add_bias', 'qil_qk_norm_rope_store',
-                 'qil_attn_rows', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_sample'):
+                 'qil_attn_rows', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_sample'):
         getattr(lib, name).restype = i

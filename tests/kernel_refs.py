@@ -72,7 +72,8 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 
 def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
-                    cu_seqlens, seq_starts, n_seqs, max_query, max_context, scale, window, accumulate=torch.float32):
+                    cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
+                    accumulate=torch.float32):
     n, d, g = qkv.shape[0], head_dim, heads // kv_heads
     q = qkv[:, :heads * d].reshape(n, heads, d).to(accumulate)
     out = torch.empty((n, heads, d), dtype=accumulate, device=qkv.device)

@@ -219,7 +219,7 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
     positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
     row_seq = torch.arange(rows, dtype=torch.int32).cuda()
     args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
-                block_tables=table, row_seq=row_seq, positions=positions, cu_seqlens=None, seq_starts=None,
+                block_tables=table, row_seq=row_seq, positions=positions, cu_seqlens=None, seq_starts=None, single_rows=None,
                 n_seqs=rows, max_query=1, max_context=max(lengths), scale=d ** -0.5, window=None)
     got = ops.paged_attention(qkv, **args)
     expected = []
@@ -240,27 +240,53 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
         torch.testing.assert_close(ops.paged_attention(qkv, **args)[0], got[0], atol=0, rtol=0)
 
 
+def mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, window, scale=0.3):
+    """Sequences of `lengths` cached tokens whose last `chunks[i]` positions are this step's rows."""
+    k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
+    starts = [n - c for n, c in zip(lengths, chunks)]
+    positions = [p for s, c in zip(starts, chunks) for p in range(s, s + c)]
+    row_seq = [i for i, c in enumerate(chunks) for _ in range(c)]
+    cu = [0]
+    for c in chunks:
+        cu.append(cu[-1] + c)
+    single = [cu[i] for i, c in enumerate(chunks) if c == 1]
+    n = cu[-1]
+    dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
+    qkv = rand(n, (heads + 2 * kv_heads) * d, dtype=dtype)
+    got = ops.paged_attention(qkv, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                              page_size=page_size, block_tables=table, row_seq=dev(row_seq), positions=dev(positions),
+                              cu_seqlens=dev(cu), seq_starts=dev(starts), single_rows=dev(single) if max(chunks) > 1 else None,
+                              n_seqs=len(lengths), max_query=max(chunks), max_context=max(lengths), scale=scale,
+                              window=window)
+    q = qkv[:, :heads * d].reshape(n, heads, d).double().cpu()
+    expected = torch.cat([
+        plain.attention(q[cu[i]:cu[i + 1]], histories[i][0].double(), histories[i][1].double(),
+                        torch.arange(starts[i], lengths[i]), scale, window)
+        for i in range(len(lengths))]).reshape(n, heads * d)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.double().cpu(), expected, **ATT_TOL[dtype])
+
+
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('window', [None, 5, 64, 300])
 def test_prompt_rows_and_window(ops, dtype, window):
     """Rows of a portion at positions 290..339 of a 340-token request beside a decoded row of another."""
-    page_size, d, heads, kv_heads = 8, 32, 6, 2
-    lengths = [340, 77]
-    k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
-    positions = torch.tensor(list(range(290, 340)) + [76], dtype=torch.int32).cuda()
-    row_seq = torch.tensor([0] * 50 + [1], dtype=torch.int32).cuda()
-    qkv = rand(51, (heads + 2 * kv_heads) * d, dtype=dtype)
-    got = ops.paged_attention(qkv, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
-                              page_size=page_size, block_tables=table, row_seq=row_seq, positions=positions,
-                              cu_seqlens=None, seq_starts=None, n_seqs=2, max_query=50, max_context=340,
-                              scale=0.3, window=window)
-    q = qkv[:, :heads * d].reshape(51, heads, d).double().cpu()
-    first = plain.attention(q[:50], histories[0][0].double(), histories[0][1].double(), positions[:50].cpu().long(),
-                            0.3, window)
-    second = plain.attention(q[50:], histories[1][0].double(), histories[1][1].double(), positions[50:].cpu().long(),
-                             0.3, window)
-    expected = torch.cat((first, second)).reshape(51, heads * d)
-    torch.testing.assert_close(got.double().cpu(), expected, **ATT_TOL[dtype])
+    mixed_attention_case(ops, dtype, [340, 77], [50, 1], 8, 32, 6, 2, window)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('lengths,chunks,page_size,d,heads,kv_heads', [
+    ([70, 70, 5, 33], [70, 2, 5, 17], 16, 128, 16, 8),          # whole prompt, two-token portion, short, middle
+    ([129, 64, 1000, 16], [129, 1, 3, 16], 16, 128, 32, 8),     # g = 4; a portion deep in a long context
+    ([257, 100], [200, 31], 3, 40, 6, 2),                       # page size 3, head size 40, g = 3
+    ([90, 45], [90, 45], 7, 256, 8, 1),                         # head size 256, one kv head (g = 8)
+    ([300, 19], [151, 19], 4, 48, 5, 1),                        # g = 5
+    ([66, 40, 20], [35, 40, 2], 8, 16, 4, 4),                   # g = 1, head size 16
+    ([513], [513], 16, 64, 4, 2),                               # g = 2
+    ([2048], [2048], 16, 128, 8, 2),
+])
+def test_prompt_portions_against_float64(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads):
+    mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, None, scale=d ** -0.5)
 
 
 def test_one_far_key_among_hundreds(ops):
@@ -276,7 +302,7 @@ def test_one_far_key_among_hundreds(ops):
         q[0, h * d:(h + 1) * d] = 200.0 * direction.cuda()
     got = ops.paged_attention(q, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
                               page_size=page_size, block_tables=table, positions=torch.tensor([n - 1], dtype=torch.int32).cuda(),
-                              row_seq=torch.zeros(1, dtype=torch.int32).cuda(), cu_seqlens=None, seq_starts=None,
+                              row_seq=torch.zeros(1, dtype=torch.int32).cuda(), cu_seqlens=None, seq_starts=None, single_rows=None,
                               n_seqs=1, max_query=1, max_context=n, scale=1.0, window=None)
     for h in range(heads):
         kvh = h // (heads // kv_heads)
