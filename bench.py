@@ -75,11 +75,13 @@ def main():
 
     def decode_run(batch):
         """(seconds per step, contexts at the middle of the timed steps) of `batch` requests decoding together."""
-        new_tokens = args.warmup + args.steps + 2
+        # requests that finish their prompt early decode while the others still prefill (about one
+        # prompt a step): leave room for that many extra tokens
+        new_tokens = args.warmup + args.steps + 2 * batch + 8
         pages = batch * (-(-(args.history + new_tokens) // page_size) + 1)
         engine = Engine(model, num_pages=pages, page_size=page_size, token_budget=args.history + batch,
                         prefill_chunk=args.history, max_active=batch)
-        ids = [engine.submit(prompt(args.history), max_new_tokens=new_tokens + batch, ignore_eos=True)
+        ids = [engine.submit(prompt(args.history), max_new_tokens=new_tokens, ignore_eos=True)
                for _ in range(batch)]
         requests = engine.scheduler.requests
         while any(requests[i].computed < args.history for i in ids):      # untimed: histories into the cache
@@ -117,12 +119,18 @@ def main():
             runner.release(attempt)
         return statistics.median(times[1:])
 
+    def note(text):
+        print(f'[bench] {text}', file=sys.stderr, flush=True)
+
     step_s, contexts = decode_run(args.batch)
+    note(f'decode batch {args.batch}: {step_s * 1e3:.3f} ms/step')
     points = {}
     for batch in [int(b) for b in args.points.split(',') if b]:
         seconds, _ = decode_run(batch)
         points[f'decode_b{batch}'] = round(batch / seconds, 1)
+        note(f'decode batch {batch}: {seconds * 1e3:.3f} ms/step')
     prefill_s = prefill_run(args.prefill_tokens)
+    note(f'prefill {args.prefill_tokens}: {prefill_s * 1e3:.2f} ms')
 
     value = args.batch / step_s
     bytes_read = decode_bytes(config, element, contexts)
