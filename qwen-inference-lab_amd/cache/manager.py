@@ -6,9 +6,10 @@ Entries with equal KV needs (kv heads, head size, window) form a group with a
 page pool of its own; every group has its own block tables, so a windowed group
 can give pages back while a full group keeps them.  Entries with equal state
 needs form a state group.  Device layout of a KV group:
-``k, v : [entries, pages, kv_heads, page_size, head_dim]`` in the model's dtype; a
-token's slot number is ``page * page_size + position % page_size``
-(qil/cache.py:79-82).  Storage is never cleared: kernels read only positions below a
+``k : [entries, pages, kv_heads, page_size, head_dim]`` and, transposed within a page so
+that the value product's matrix-core operands load directly,
+``v : [entries, pages, kv_heads, head_dim, page_size]``, in the model's dtype; a token's slot
+number is ``page * page_size + position % page_size`` (qil/cache.py:79-82).  Storage is never cleared: kernels read only positions below a
 request's computed length and inside its window (qil/cache.py:127-128,137;
 tests fill the pool with NaN).
 
@@ -29,7 +30,7 @@ from .pages import PagePool, CacheFull
 class KVView:
     """What an attention-like mixer sees of its schedule entry's cache in one step."""
     k: torch.Tensor              # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor              # [pages, kv_heads, head_dim, page_size]
     page_size: int
     writes: bool                 # False for an entry that reads another entry's cache
     group: int
@@ -89,9 +90,11 @@ class CacheManager:
     def _allocate(self):
         for group in self.kv_groups:
             need, pool = group['need'], group['pool']
-            shape = (len(group['entries']), pool.capacity, need.kv_heads, self.page_size, need.head_dim)
-            group['k'] = torch.empty(shape, dtype=self.dtype, device=self.device)
-            group['v'] = torch.empty(shape, dtype=self.dtype, device=self.device)
+            entries, pages = len(group['entries']), pool.capacity
+            group['k'] = torch.empty((entries, pages, need.kv_heads, self.page_size, need.head_dim),
+                                     dtype=self.dtype, device=self.device)
+            group['v'] = torch.empty((entries, pages, need.kv_heads, need.head_dim, self.page_size),
+                                     dtype=self.dtype, device=self.device)
         for group in self.state_groups:
             need = group['need']
             dtype = torch.float32 if need.dtype == 'float32' else self.dtype

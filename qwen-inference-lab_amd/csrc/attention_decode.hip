@@ -1,0 +1,233 @@
+// Split-context attention of single rows (decoded tokens) on the matrix cores, bfloat16.
+//
+// Same task and the same partial results as the row kernel in attention_rows.hip (a block owns
+// the keys [part * P, (part + 1) * P) of one row and one kv head and serves the whole group of
+// query heads reading that kv head; the merge kernel there combines the parts), but the operands
+// go from global memory straight into v_mfma_f32_16x16x32_bf16, with no staging in LDS:
+//
+//   S^T[key, head] = sum_dim K[key, dim] Q[head, dim]     A = K rows      (K is [.., page_size, d])
+//   O^T[dim, head] = sum_key V^T[dim, key] P^T[key, head] A = V^T rows    (V is [.., d, page_size])
+//
+// The 16 columns of a tile are the g query heads of the kv head (columns from g on are zero), so
+// a lane holds the scores of ONE head for keys 4 (lane / 16) + i, and softmax statistics are
+// per-lane scalars reduced over the 4 lane groups by two shuffles (qil/paged_attention.py:27-41
+// computes the same maxima, sums and weighted values in float32).  Each of the block's 4 waves
+// takes every fourth 32-key step and keeps its own running (m, l, O); the four meet in LDS once.
+//
+// Invisible keys (j > position, or outside the window) may lie in pages that were never
+// written or belong to someone else: their scores are replaced, not multiplied, and their V
+// elements are zeroed before the product, so garbage (even NaN) cannot enter a sum.
+//
+// Takes page_size % 4 == 0, d % 16 == 0, d <= 256, g <= 16; other sizes go to the row kernel.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define DEC_THREADS 256
+#define DEC_WAVES 4
+
+template <int DMAX>
+__global__ void __launch_bounds__(DEC_THREADS)
+attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                   const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
+                   const int* __restrict__ row_seq, const int* __restrict__ positions,
+                   const int* __restrict__ row_index, float* __restrict__ part_acc, float* __restrict__ part_m,
+                   float* __restrict__ part_l, bf16_t* __restrict__ out, int heads, int kv_heads, int d,
+                   int page_size, int window, float scale, int P, int parts) {
+  constexpr int QFRAGS = DMAX / 32, DTILES = DMAX / 16;
+  extern __shared__ float lds[];
+  const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
+  const int row = row_index ? row_index[slot_row] : slot_row;
+  const int g = heads / kv_heads;
+  const int pos = positions[row], ctx = pos + 1;
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int begin = max(part * P, lo), end = min((part + 1) * P, ctx);
+  if (begin >= end) return;
+
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int dt = d / 16;
+  const int* table = block_tables + (size_t)row_seq[row] * table_stride;
+
+  // Q fragments: B operand, column r = head kvh * g + r
+  bf16x8 qb[QFRAGS];
+#pragma unroll
+  for (int ks = 0; ks < QFRAGS; ++ks) {
+    const int dim = ks * 32 + kb * 8;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (r < g && dim < d) raw = *reinterpret_cast<const uint4*>(q + (size_t)row * q_stride + (size_t)(kvh * g + r) * d + dim);
+    qb[ks] = __builtin_bit_cast(bf16x8, raw);
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[DTILES];
+#pragma unroll
+  for (int t = 0; t < DTILES; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int first_step = begin / 32;                       // 32-key steps, absolute numbering
+  const int last_step = (end - 1) / 32;
+  for (int step = first_step + wave; step <= last_step; step += DEC_WAVES) {
+    const int k0 = step * 32;
+    // ---- loads first: K rows of both 16-key sub-tiles, then the V^T fragments of every dim tile
+    uint4 kraw[2][QFRAGS];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+      const int key = min(k0 + jt * 16 + r, ctx - 1);      // clamped: an invisible key's score is replaced below
+      const size_t page = table[key / page_size];
+      const bf16_t* krow = k_cache + ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d;
+#pragma unroll
+      for (int ks = 0; ks < QFRAGS; ++ks) {
+        const int dim = ks * 32 + kb * 8;
+        kraw[jt][ks] = (ks * 32 < d && dim < d) ? *reinterpret_cast<const uint4*>(krow + dim) : make_uint4(0, 0, 0, 0);
+      }
+    }
+    uint2 vraw[DTILES][2];
+    {
+      const bf16_t* vbase[2];
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const int key = min(k0 + hf * 16 + 4 * kb, ctx - 1) & ~3;    // group of 4 keys inside one page
+        const size_t page = table[key / page_size];
+        vbase[hf] = v_cache + (page * kv_heads + kvh) * (size_t)d * page_size + (key % page_size);
+      }
+#pragma unroll
+      for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+          vraw[t][hf] = t < dt ? *reinterpret_cast<const uint2*>(vbase[hf] + (size_t)(t * 16 + r) * page_size)
+                               : make_uint2(0, 0);
+    }
+    // ---- scores
+    f32x4 s[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < QFRAGS; ++ks)
+        if (ks * 32 < d) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kraw[jt][ks]), qb[ks], acc, 0, 0, 0);
+      s[jt] = acc;
+    }
+    float mx = -INFINITY;
+    uint32_t keep[2][4];                                    // 0xffff where the key is visible
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + jt * 16 + 4 * kb + i;
+        const bool visible = key >= begin && key < end;
+        keep[jt][i] = visible ? 0xffffu : 0u;
+        const float v = visible ? s[jt][i] * scale : -INFINITY;
+        s[jt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * 1.44269504088896f);
+    float psum = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = (s[jt][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((s[jt][i] - m_new) * 1.44269504088896f);
+        s[jt][i] = p;
+        psum += p;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // ---- O^T = O^T alpha + V^T P^T
+    uint32_t packed[4];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        packed[jt * 2 + i] = (uint32_t)f32_to_bf16(s[jt][2 * i]) | ((uint32_t)f32_to_bf16(s[jt][2 * i + 1]) << 16);
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+    const uint32_t mask[4] = {keep[0][0] | (keep[0][1] << 16), keep[0][2] | (keep[0][3] << 16),
+                              keep[1][0] | (keep[1][1] << 16), keep[1][2] | (keep[1][3] << 16)};
+#pragma unroll
+    for (int t = 0; t < DTILES; ++t) {
+      if (t < dt) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vraw[t][0].x & mask[0], vraw[t][0].y & mask[1],
+                                                                vraw[t][1].x & mask[2], vraw[t][1].y & mask[3]));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- the four waves' (m, l, O) meet in LDS: [wave][head < g][d + 2]
+  l += __shfl_xor(l, 16, QIL_WAVE);
+  l += __shfl_xor(l, 32, QIL_WAVE);
+  const int cell = d + 2;
+  if (r < g) {
+    float* mine = lds + ((size_t)wave * g + r) * cell;
+    if (kb == 0) { mine[d] = m; mine[d + 1] = l; }
+#pragma unroll
+    for (int t = 0; t < DTILES; ++t)
+      if (t < dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine[t * 16 + 4 * kb + i] = o[t][i];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < g * d; idx += DEC_THREADS) {
+    const int h = idx / d, e = idx - h * d;
+    float mw[DEC_WAVES], mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      mw[w] = lds[((size_t)w * g + h) * cell + d];
+      mm = fmaxf(mm, mw[w]);
+    }
+    float total = 0.f, ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float f = mw[w] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mw[w] - mm) * 1.44269504088896f);
+      total += lds[((size_t)w * g + h) * cell + e] * f;
+      ll += lds[((size_t)w * g + h) * cell + d + 1] * f;
+    }
+    const int head = kvh * g + h;
+    if (parts == 1) {
+      out[((size_t)row * heads + head) * d + e] = f32_to_bf16(total / ll);
+    } else {
+      const size_t c = ((size_t)slot_row * heads + head) * parts + part;
+      part_acc[c * d + e] = total;
+      if (e == 0) { part_m[c] = mm; part_l[c] = ll; }
+    }
+  }
+}
+
+// 1 if the matrix-core decode kernel takes these sizes.
+extern "C" int qil_attn_decode_takes(int heads, int kv_heads, int d, int page_size) {
+  if (heads % kv_heads || d % 16 || d < 16 || d > 256 || page_size % 4) return 0;
+  const int g = heads / kv_heads;
+  return g <= 16 && (size_t)DEC_WAVES * g * (d + 2) * sizeof(float) <= 64 * 1024;
+}
+
+// Partial results in the layout of the row kernel (acc [rows, heads, parts, d], then m, then l);
+// the caller runs the row kernel's merge when parts > 1.  P must be a multiple of 32.
+extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                               const int* block_tables, int table_stride, const int* row_seq, const int* positions,
+                               const int* row_index, void* workspace, void* out, int rows, int heads, int kv_heads,
+                               int d, int page_size, int window, float scale, int P, int parts, hipStream_t s) {
+  if (rows == 0) return 0;
+  if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || P % 32 || P < 32 || parts < 1 || parts > 65535 ||
+      kv_heads > 65535)
+    return -1;
+  const int g = heads / kv_heads;
+  float* acc = (float*)workspace;
+  float* m = acc ? acc + (size_t)rows * heads * parts * d : nullptr;
+  float* l = m ? m + (size_t)rows * heads * parts : nullptr;
+  const size_t lds = (size_t)DEC_WAVES * g * (d + 2) * sizeof(float);
+  dim3 grid(rows, kv_heads, parts);
+#define QIL_DEC_CASE(DMAX)                                                                                          \
+  hipLaunchKernelGGL(attn_decode_kernel<DMAX>, grid, dim3(DEC_THREADS), lds, s, (const bf16_t*)q, q_stride,          \
+                     (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
+                     row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts)
+  if (d <= 64) QIL_DEC_CASE(64);
+  else if (d <= 128) QIL_DEC_CASE(128);
+  else QIL_DEC_CASE(256);
+#undef QIL_DEC_CASE
+  QIL_RETURN_LAUNCH_STATUS();
+}

@@ -113,12 +113,11 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
     for (int t = wave * TPW + slot; t < count; t += ATT_WAVES * TPW) {
       const int j = begin + t;
       const size_t page = table[j / page_size];
-      const size_t base = ((page * kv_heads + kvh) * page_size + (j % page_size)) * (size_t)d + e0;
+      // V is [pages, kv_heads, d, page_size]: this key's elements lie page_size apart
+      const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + e0) * page_size + (j % page_size);
       float vv[8];
-      if (live) ld8(v_cache + base, vv);
-      else
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vv[e] = 0.f;
+      for (int e = 0; e < 8; ++e) vv[e] = live ? ld(column + (size_t)e * page_size) : 0.f;
 #pragma unroll
       for (int h = 0; h < GT; ++h) {
         const float p = scores[h * P + t];
@@ -254,6 +253,23 @@ int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* 
                               acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
   return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+}
+
+// Merge of partial results written by a partial kernel (this file's or the matrix-core decode kernel's).
+int qil_attn_merge(const void* workspace, const int* positions, const int* row_index, void* out, int rows, int heads,
+                   int d, int window, int P, int parts, int dtype, hipStream_t s) {
+  if (rows == 0 || parts <= 1) return 0;
+  const float* acc = (const float*)workspace;
+  const float* m = acc + (size_t)rows * heads * parts * d;
+  const float* l = m + (size_t)rows * heads * parts;
+  const dim3 grid(rows, heads), block(d >= 128 ? 128 : 64);
+  if (dtype == QIL_F32)
+    hipLaunchKernelGGL(attn_rows_merge_kernel<float>, grid, block, 0, s, acc, m, l, positions, row_index, (float*)out,
+                       heads, d, window, P, parts);
+  else
+    hipLaunchKernelGGL(attn_rows_merge_kernel<bf16_t>, grid, block, 0, s, acc, m, l, positions, row_index, (bf16_t*)out,
+                       heads, d, window, P, parts);
+  QIL_RETURN_LAUNCH_STATUS();
 }
 
 }  // extern "C"

@@ -131,7 +131,11 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
           const size_t page = table[key / page_size];
           const size_t base = ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d + dv;
           kraw = *reinterpret_cast<const uint4*>(k_cache + base);
-          vraw = *reinterpret_cast<const uint4*>(v_cache + base);
+          const bf16_t* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + dv) * page_size + (key % page_size);
+          uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e >> 1] |= (uint32_t)column[(size_t)e * page_size] << ((e & 1) * 16);
+          vraw = make_uint4(w[0], w[1], w[2], w[3]);
         }
         *reinterpret_cast<uint4*>(kdst) = kraw;
         const uint32_t w[4] = {vraw.x, vraw.y, vraw.z, vraw.w};
@@ -145,7 +149,9 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
           const size_t page = table[key / page_size];
           const size_t base = ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d + dv;
           ld8(k_cache + base, kv8);
-          ld8(v_cache + base, vv8);
+          const float* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + dv) * page_size + (key % page_size);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vv8[e] = column[(size_t)e * page_size];
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) { kdst[e] = kv8[e]; Vt[(dv + e) * v_row + kl] = vv8[e]; }

@@ -12,24 +12,44 @@ __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
 }
 
+// A sub-layer's output arrives either in the model's type T (one array) or as float32 partial sums
+// of a K-split matrix product, [splits][rows][width], which the consumer adds in split order.
+template <typename TD>
+__device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t index, int splits, size_t stride) {
+  float v = ld(base + index);
+  for (int s = 1; s < splits; ++s) v += ld(base + s * stride + index);
+  return v;
+}
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                     __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2((uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
+                                            (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16));
+}
+
 // One block per output row.
 //   x = stream[r] (+ delta[r]);  if (update) stream[r] = x;
 //   out[m] = round_T(round_T(x * rsqrt(mean(x^2) + eps)) * weight)   (qil/model.py:15-23)
 // r = rows ? rows[m] : m.  Statistics, the sum and the weight product are float32.
-template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
-                                   const int* __restrict__ rows, const float* __restrict__ weight,
-                                   T* __restrict__ out, int width, float eps, int update) {
+template <typename TD, typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ stream, const TD* __restrict__ delta, int splits,
+                                   size_t split_stride, const int* __restrict__ rows,
+                                   const float* __restrict__ weight, T* __restrict__ out, int width, float eps,
+                                   int update) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
   const size_t r = rows ? (size_t)rows[m] : (size_t)m;
   float* x = stream + r * width;
-  const T* d = delta ? delta + r * width : nullptr;
   float sum = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = x[i];
-    if (d) {
-      v += ld(d + i);
+    if (delta) {
+      v += load_sum(delta, r * width + i, splits, split_stride);
       if (update) x[i] = v;
     }
     sum += v * v;
@@ -39,20 +59,64 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restri
   T* y = out + (size_t)m * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = x[i];
-    if (d && !update) v += ld(d + i);
+    if (delta && !update) v += load_sum(delta, r * width + i, splits, split_stride);
     st(y + i, round_to<T>(v * rstd) * weight[i]);
   }
 }
 
+// The same for width % 4 == 0 and width <= 16 * THREADS: the row stays in registers between the
+// two passes and every access is a 16-byte (8-byte for bfloat16) vector.
+template <typename TD, typename T, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+add_rmsnorm_vec_kernel(float* __restrict__ stream, const TD* __restrict__ delta, int splits, size_t split_stride,
+                       const int* __restrict__ rows, const float* __restrict__ weight, T* __restrict__ out, int width,
+                       float eps, int update) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const size_t r = rows ? (size_t)rows[m] : (size_t)m;
+  float* x = stream + r * width;
+  float4 cache[4];
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (threadIdx.x + j * THREADS) * 4;
+    if (i < width) {
+      float4 v = load4(x + i);
+      if (delta) {
+        for (int s = 0; s < splits; ++s) {
+          const float4 d = load4(delta + s * split_stride + r * width + i);
+          v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        if (update) store4(x + i, v);
+      }
+      cache[j] = v;
+      sum += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+  }
+  sum = block_sum(sum, scratch);
+  const float rstd = rsqrtf(sum / (float)width + eps);
+  T* y = out + (size_t)m * width;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (threadIdx.x + j * THREADS) * 4;
+    if (i < width) {
+      const float4 v = cache[j], w = load4(weight + i);
+      store4(y + i, make_float4(round_to<T>(v.x * rstd) * w.x, round_to<T>(v.y * rstd) * w.y,
+                                round_to<T>(v.z * rstd) * w.z, round_to<T>(v.w * rstd) * w.w));
+    }
+  }
+}
+
 // out[n, i] = silu(gate_up[n, i]) * gate_up[n, inner + i], silu(z) = z * sigmoid(z)   (qil/model.py:71)
-template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inner, size_t total) {
+template <typename TD, typename T>
+__global__ void silu_mul_kernel(const TD* __restrict__ gate_up, int splits, size_t split_stride, T* __restrict__ out,
+                                int inner, size_t total) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t n = idx / inner;
   const int i = (int)(idx - n * inner);
-  const float g = ld(gate_up + n * 2 * (size_t)inner + i);
-  const float u = ld(gate_up + n * 2 * (size_t)inner + inner + i);
+  const float g = load_sum(gate_up, n * 2 * (size_t)inner + i, splits, split_stride);
+  const float u = load_sum(gate_up, n * 2 * (size_t)inner + inner + i, splits, split_stride);
   st(out + idx, (g / (1.f + expf(-g))) * u);
 }
 
@@ -76,27 +140,59 @@ int qil_embed(const int* tokens, const void* table, float* stream, int n, int wi
   QIL_RETURN_LAUNCH_STATUS();
 }
 
-int qil_add_rmsnorm(float* stream, const void* delta, const int* rows, const float* weight, void* out,
-                    int n_out, int width, float eps, int update, int dtype, hipStream_t s) {
+// delta: null, or the sub-layer output to add: delta_dtype QIL_BF16 (one array, splits == 1) or QIL_F32
+// ([splits][delta_rows][width] partial sums).  out_dtype: type of `out`.
+int qil_add_rmsnorm(float* stream, const void* delta, int delta_dtype, int splits, int delta_rows, const int* rows,
+                    const float* weight, void* out, int n_out, int width, float eps, int update, int out_dtype,
+                    hipStream_t s) {
   if (n_out == 0) return 0;
-  const int threads = width >= 2048 ? 512 : width >= 512 ? 256 : 64;
-  if (dtype == QIL_F32)
-    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, s, stream, (const float*)delta,
-                       rows, weight, (float*)out, width, eps, update);
-  else
-    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_out), dim3(threads), 0, s, stream, (const bf16_t*)delta,
-                       rows, weight, (bf16_t*)out, width, eps, update);
+  if (splits < 1 || (delta_dtype == QIL_BF16 && splits != 1)) return -1;
+  const size_t stride = (size_t)delta_rows * width;
+  const bool vec = width % 4 == 0 && width <= 16 * 256 &&
+                   (((uintptr_t)stream | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) % 16 == 0);
+#define QIL_NORM_CASE(TD, T)                                                                                         \
+  do {                                                                                                               \
+    if (vec && width <= 16 * 64)                                                                                     \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, T, 64>), dim3(n_out), dim3(64), 0, s, stream, (const TD*)delta, \
+                         splits, stride, rows, weight, (T*)out, width, eps, update);                                 \
+    else if (vec)                                                                                                    \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, T, 256>), dim3(n_out), dim3(256), 0, s, stream,                 \
+                         (const TD*)delta, splits, stride, rows, weight, (T*)out, width, eps, update);               \
+    else                                                                                                             \
+      hipLaunchKernelGGL((add_rmsnorm_kernel<TD, T>), dim3(n_out), dim3(width >= 2048 ? 512 : width >= 512 ? 256 : 64), \
+                         0, s, stream, (const TD*)delta, splits, stride, rows, weight, (T*)out, width, eps, update); \
+  } while (0)
+  if (out_dtype == QIL_F32) {
+    if (delta_dtype != QIL_F32) return -1;
+    QIL_NORM_CASE(float, float);
+  } else if (delta_dtype == QIL_F32) {
+    QIL_NORM_CASE(float, bf16_t);
+  } else {
+    QIL_NORM_CASE(bf16_t, bf16_t);
+  }
+#undef QIL_NORM_CASE
   QIL_RETURN_LAUNCH_STATUS();
 }
 
-int qil_silu_mul(const void* gate_up, void* out, int n, int inner, int dtype, hipStream_t s) {
+// gate_up: in_dtype QIL_BF16 [n, 2 inner] or QIL_F32 [splits][n][2 inner] partial sums.
+int qil_silu_mul(const void* gate_up, int in_dtype, int splits, void* out, int n, int inner, int out_dtype,
+                 hipStream_t s) {
   const size_t total = (size_t)n * inner;
   if (total == 0) return 0;
+  if (splits < 1 || (in_dtype == QIL_BF16 && splits != 1)) return -1;
+  const size_t stride = (size_t)n * 2 * inner;
   const unsigned blocks = (unsigned)((total + 255) / 256);
-  if (dtype == QIL_F32)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gate_up, (float*)out, inner, total);
-  else
-    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gate_up, (bf16_t*)out, inner, total);
+  if (out_dtype == QIL_F32) {
+    if (in_dtype != QIL_F32) return -1;
+    hipLaunchKernelGGL((silu_mul_kernel<float, float>), dim3(blocks), dim3(256), 0, s, (const float*)gate_up, splits,
+                       stride, (float*)out, inner, total);
+  } else if (in_dtype == QIL_F32) {
+    hipLaunchKernelGGL((silu_mul_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, s, (const float*)gate_up, splits,
+                       stride, (bf16_t*)out, inner, total);
+  } else {
+    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, s, (const bf16_t*)gate_up, splits,
+                       stride, (bf16_t*)out, inner, total);
+  }
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -21,53 +21,99 @@ __device__ __forceinline__ float gumbel(uint32_t seed, uint32_t counter, uint32_
   return -logf(-logf(u));
 }
 
-#define SAMPLE_THREADS 512
+#define SAMPLE_THREADS 256
+#define SAMPLE_CHUNK 4096          // vocabulary entries per first-stage block
 
+struct Best { float value; int index; int broken; };
+
+// Larger value wins; on equal values the lower index (argmax's tie rule, qil/engine.py:100).
+__device__ __forceinline__ void take(Best& a, float value, int index) {
+  if (value > a.value || (value == a.value && index < a.index)) { a.value = value; a.index = index; }
+}
+
+__device__ __forceinline__ Best block_best(Best mine, float* values, int* indices, int* bad) {
+  for (int o = QIL_WAVE / 2; o > 0; o >>= 1) {
+    const float v = __shfl_xor(mine.value, o, QIL_WAVE);
+    const int i = __shfl_xor(mine.index, o, QIL_WAVE);
+    mine.broken |= __shfl_xor(mine.broken, o, QIL_WAVE);
+    take(mine, v, i);
+  }
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  if (lane == 0) { values[wave] = mine.value; indices[wave] = mine.index; bad[wave] = mine.broken; }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int w = 1; w < (int)(blockDim.x / QIL_WAVE); ++w) {
+      mine.broken |= bad[w];
+      take(mine, values[w], indices[w]);
+    }
+  return mine;                       // complete in thread 0
+}
+
+// Stage 1: grid (chunks, rows).  Each block scans SAMPLE_CHUNK logits of one row.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
-              const int* __restrict__ seeds, const int* __restrict__ counters, int* __restrict__ tokens,
-              int* __restrict__ finite, int vocab) {
-  __shared__ float best_value[SAMPLE_THREADS / QIL_WAVE];
-  __shared__ int best_index[SAMPLE_THREADS / QIL_WAVE];
-  __shared__ int bad[SAMPLE_THREADS / QIL_WAVE];
-  const int row = blockIdx.x;
+sample_scan_kernel(const float* __restrict__ logits, const float* __restrict__ temperatures,
+                   const int* __restrict__ seeds, const int* __restrict__ counters, float* __restrict__ chunk_value,
+                   int* __restrict__ chunk_index, int* __restrict__ chunk_bad, int vocab, int chunks) {
+  __shared__ float values[SAMPLE_THREADS / QIL_WAVE];
+  __shared__ int indices[SAMPLE_THREADS / QIL_WAVE], bad[SAMPLE_THREADS / QIL_WAVE];
+  const int chunk = blockIdx.x, row = blockIdx.y;
   const float* x = logits + (size_t)row * vocab;
   const float temperature = temperatures[row];
   const uint32_t seed = (uint32_t)seeds[row], counter = (uint32_t)counters[row];
-  float value = -INFINITY;
-  int index = 0x7fffffff, broken = 0;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+  Best mine = {-INFINITY, 0x7fffffff, 0};
+  const int stop = min(vocab, (chunk + 1) * SAMPLE_CHUNK);
+  for (int i = chunk * SAMPLE_CHUNK + threadIdx.x; i < stop; i += SAMPLE_THREADS) {
     const float v = x[i];
-    if (!isfinite(v)) broken = 1;
-    const float score = temperature > 0.f ? v / temperature + gumbel(seed, counter, (uint32_t)i) : v;
-    if (score > value) { value = score; index = i; }          // strided ascending: first maximum kept
+    if (!isfinite(v)) mine.broken = 1;
+    take(mine, temperature > 0.f ? v / temperature + gumbel(seed, counter, (uint32_t)i) : v, i);
   }
-  for (int o = QIL_WAVE / 2; o > 0; o >>= 1) {
-    const float other = __shfl_xor(value, o, QIL_WAVE);
-    const int other_index = __shfl_xor(index, o, QIL_WAVE);
-    broken |= __shfl_xor(broken, o, QIL_WAVE);
-    if (other > value || (other == value && other_index < index)) { value = other; index = other_index; }
-  }
-  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
-  if (lane == 0) { best_value[wave] = value; best_index[wave] = index; bad[wave] = broken; }
-  __syncthreads();
+  mine = block_best(mine, values, indices, bad);
   if (threadIdx.x == 0) {
-    for (int w = 1; w < SAMPLE_THREADS / QIL_WAVE; ++w) {
-      broken |= bad[w];
-      if (best_value[w] > value || (best_value[w] == value && best_index[w] < index)) {
-        value = best_value[w];
-        index = best_index[w];
-      }
-    }
-    tokens[row] = index == 0x7fffffff ? 0 : index;
-    finite[row] = broken ? 0 : 1;
+    const size_t cell = (size_t)row * chunks + chunk;
+    chunk_value[cell] = mine.value; chunk_index[cell] = mine.index; chunk_bad[cell] = mine.broken;
   }
 }
 
-extern "C" int qil_sample(const float* logits, const float* temperatures, const int* seeds, const int* counters,
-                          int* tokens, int* finite, int rows, int vocab, hipStream_t s) {
+// Stage 2: one block per row over the chunks' winners.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_pick_kernel(const float* __restrict__ chunk_value, const int* __restrict__ chunk_index,
+                   const int* __restrict__ chunk_bad, int* __restrict__ tokens, int* __restrict__ finite, int chunks) {
+  __shared__ float values[SAMPLE_THREADS / QIL_WAVE];
+  __shared__ int indices[SAMPLE_THREADS / QIL_WAVE], bad[SAMPLE_THREADS / QIL_WAVE];
+  const int row = blockIdx.x;
+  Best mine = {-INFINITY, 0x7fffffff, 0};
+  for (int c = threadIdx.x; c < chunks; c += SAMPLE_THREADS) {
+    const size_t cell = (size_t)row * chunks + c;
+    mine.broken |= chunk_bad[cell];
+    take(mine, chunk_value[cell], chunk_index[cell]);
+  }
+  mine = block_best(mine, values, indices, bad);
+  if (threadIdx.x == 0) {
+    tokens[row] = mine.index == 0x7fffffff ? 0 : mine.index;
+    finite[row] = mine.broken ? 0 : 1;
+  }
+}
+
+extern "C" {
+
+// Bytes of scratch for `rows` rows: per chunk a value, an index and a flag.
+size_t qil_sample_workspace(int rows, int vocab) {
+  return (size_t)rows * ((vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK) * 12;
+}
+
+int qil_sample(const float* logits, const float* temperatures, const int* seeds, const int* counters, int* tokens,
+               int* finite, void* workspace, int rows, int vocab, hipStream_t s) {
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, s, logits, temperatures, seeds, counters,
-                     tokens, finite, vocab);
+  if (rows > 65535) return -1;
+  const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  float* values = (float*)workspace;
+  int* indices = (int*)(values + (size_t)rows * chunks);
+  int* bad = indices + (size_t)rows * chunks;
+  hipLaunchKernelGGL(sample_scan_kernel, dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, s, logits, temperatures, seeds,
+                     counters, values, indices, bad, vocab, chunks);
+  hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, s, values, indices, bad, tokens, finite,
+                     chunks);
   QIL_RETURN_LAUNCH_STATUS();
 }
+
+}  // extern "C"

@@ -22,7 +22,7 @@ def _full_attention(config, rotary, dtype):
 
 
 def _dense_mlp(config, dtype):
-    return GatedMLP(width=config.hidden_size, intermediate=config.intermediate_size, activation='silu')
+    return GatedMLP(width=config.hidden_size, intermediate=config.intermediate_size, activation='silu', dtype=dtype)
 
 
 # Layer kinds this architecture can hold, chosen layer by layer.

@@ -19,10 +19,33 @@ from . import library
 STREAM_GEMM_MAX_ROWS = 64
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
+# Blocks the matrix-core decode kernel aims for (256 CUs).
+DECODE_BLOCKS = 1024
 
 
 class UnsupportedShape(ValueError):
     pass
+
+
+class Partials:
+    """A matrix product left as float32 partial sums [splits, N, O]; its value is their sum in split
+    order, made by the kernel that consumes it (norm, rotary/store, SiLU gate)."""
+
+    def __init__(self, tensor):
+        self.tensor, self.splits, self.shape = tensor, tensor.shape[0], tuple(tensor.shape[1:])
+        self.device = tensor.device
+
+    def sum(self):
+        return self.tensor.sum(dim=0)
+
+
+def _operand(value, name, model_dtype, shape):
+    """(pointer, dtype code, splits) of a consumer's input: a tensor of the model's type or Partials."""
+    if isinstance(value, Partials):
+        _require(value.tensor, name, torch.float32, (value.splits, *shape))
+        return value.tensor.data_ptr(), 0, value.splits
+    _require(value, name, model_dtype, shape)
+    return value.data_ptr(), _code(model_dtype), 1
 
 
 _CODES = {torch.float32: 0, torch.bfloat16: 1}
@@ -69,6 +92,17 @@ def check_attention_geometry(*, heads, kv_heads, head_dim, dtype):
         raise UnsupportedShape(f'head_dim {head_dim}: the attention kernels take multiples of 8 from 8 to 256')
 
 
+def _check_caches(k_cache, v_cache, dtype, kv_heads, page_size, head_dim):
+    """K [pages, kv_heads, page_size, d]; V transposed within the page: [pages, kv_heads, d, page_size]."""
+    _require(k_cache, 'k_cache', dtype)
+    _require(v_cache, 'v_cache', dtype)
+    if k_cache.ndim != 4 or tuple(k_cache.shape[1:]) != (kv_heads, page_size, head_dim):
+        raise ValueError(f'k_cache must be [pages, {kv_heads}, {page_size}, {head_dim}]')
+    if v_cache.ndim != 4 or tuple(v_cache.shape[1:]) != (kv_heads, head_dim, page_size) \
+            or v_cache.shape[0] != k_cache.shape[0]:
+        raise ValueError(f'v_cache must be [pages, {kv_heads}, {head_dim}, {page_size}]')
+
+
 def embed(token_ids, table):
     """int32 [N], T [V, H] -> float32 stream [N, H]."""
     _require(token_ids, 'token_ids', torch.int32)
@@ -81,15 +115,16 @@ def embed(token_ids, table):
 
 
 def add_rmsnorm(stream, delta, weight, eps, out_dtype):
-    """stream += delta (in place, float32 sum; skipped if delta is None); returns norm(stream) as out_dtype."""
+    """stream += delta (in place, float32 sum; skipped if delta is None); returns norm(stream) as out_dtype.
+
+    ``delta``: tensor of ``out_dtype`` [N, H] or Partials."""
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
-    if delta is not None:
-        _require(delta, 'delta', out_dtype, (n, width))
+    pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
     out = torch.empty((n, width), dtype=out_dtype, device=stream.device)
-    _check(library.load().qil_add_rmsnorm(_ptr(stream), _ptr(delta), None, _ptr(weight), _ptr(out), n, width,
-                                          float(eps), 1, _code(out_dtype), _stream()), 'add_rmsnorm')
+    _check(library.load().qil_add_rmsnorm(_ptr(stream), pointer, code, splits, n, None, _ptr(weight), _ptr(out), n,
+                                          width, float(eps), 1, _code(out_dtype), _stream()), 'add_rmsnorm')
     return out
 
 
@@ -99,17 +134,19 @@ def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
     _require(rows, 'rows', torch.int32)
-    if delta is not None:
-        _require(delta, 'delta', out_dtype, (n, width))
+    pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
     out = torch.empty((rows.shape[0], width), dtype=out_dtype, device=stream.device)
-    _check(library.load().qil_add_rmsnorm(_ptr(stream), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out),
+    _check(library.load().qil_add_rmsnorm(_ptr(stream), pointer, code, splits, n, _ptr(rows), _ptr(weight), _ptr(out),
                                           rows.shape[0], width, float(eps), 0, _code(out_dtype), _stream()),
            'rows_rmsnorm')
     return out
 
 
-def linear(x, weight, bias=None, out_dtype=None):
-    """x [N, K] @ weight [O, K]^T (+ bias float32 [O]) -> [N, O] in out_dtype (default: x's)."""
+def linear(x, weight, bias=None, out_dtype=None, partials=False):
+    """x [N, K] @ weight [O, K]^T (+ bias float32 [O]) -> [N, O] in out_dtype (default: x's).
+
+    ``partials=True`` allows the result to come back as ``Partials`` (bfloat16 products with few
+    rows: float32, K split over blocks) for a consumer that adds them; otherwise a tensor."""
     _require(x, 'x')
     _require(weight, 'weight', x.dtype)
     n, k = x.shape
@@ -127,10 +164,15 @@ def linear(x, weight, bias=None, out_dtype=None):
         _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _stream()), 'gemm_f32')
         return out
     _code(x.dtype)
+    if n <= STREAM_GEMM_MAX_ROWS and partials and bias is None and out_dtype == x.dtype:
+        splits = lib.qil_gemm_bf16_splits(n, o, k)
+        out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, _stream()), 'gemm_bf16')
+        return Partials(out)
     if out_dtype == torch.float32 or n <= STREAM_GEMM_MAX_ROWS:
         out = torch.empty((n, o), dtype=out_dtype, device=x.device)
-        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), _stream()),
-               'gemm_bf16')
+        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), 1,
+                                 _stream()), 'gemm_bf16')
         return out
     out = torch.mm(x, weight.t())                      # GPU BLAS, float32 accumulation
     if bias is not None:
@@ -138,24 +180,29 @@ def linear(x, weight, bias=None, out_dtype=None):
     return out
 
 
-def silu_mul(gate_up):
-    """T [N, 2 I] (gate columns first) -> silu(gate) * up, T [N, I]."""
-    _require(gate_up, 'gate_up')
+def silu_mul(gate_up, out_dtype=None):
+    """[N, 2 I] (gate columns first; tensor of the model's type or Partials) -> silu(gate) * up, [N, I]."""
     n, both = gate_up.shape
     if both % 2:
         raise ValueError('silu_mul: needs an even number of columns')
-    out = torch.empty((n, both // 2), dtype=gate_up.dtype, device=gate_up.device)
-    _check(library.load().qil_silu_mul(_ptr(gate_up), _ptr(out), n, both // 2, _code(gate_up.dtype), _stream()),
+    out_dtype = out_dtype or (gate_up.dtype if not isinstance(gate_up, Partials) else None)
+    if out_dtype is None:
+        raise ValueError('silu_mul of Partials needs out_dtype')
+    pointer, code, splits = _operand(gate_up, 'gate_up', out_dtype, (n, both))
+    out = torch.empty((n, both // 2), dtype=out_dtype, device=gate_up.device)
+    _check(library.load().qil_silu_mul(pointer, code, splits, _ptr(out), n, both // 2, _code(out_dtype), _stream()),
            'silu_mul')
     return out
 
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size):
-    """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given); q back
-    into ``qkv`` in place, k and v into the caches at ``slots`` (None: not stored)."""
+                       k_cache, v_cache, page_size, dtype):
+    """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given).
+
+    ``qkv`` [N, (heads + 2 kv_heads) d]: tensor of type ``dtype`` or Partials.  Returns q as ``dtype``
+    [N, heads * d]; k and v go into the caches at ``slots`` (None: not stored)."""
     n = qkv.shape[0]
-    _require(qkv, 'qkv', None, (n, (heads + 2 * kv_heads) * head_dim))
+    pointer, code, splits = _operand(qkv, 'qkv', dtype, (n, (heads + 2 * kv_heads) * head_dim))
     _require(positions, 'positions', torch.int32, (n,))
     for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
         if w is not None:
@@ -172,38 +219,34 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
             raise ValueError('rotation tables do not fit rot_dim')
     if slots is not None:
         _require(slots, 'slots', torch.int32, (n,))
-        for cache, name in ((k_cache, 'k_cache'), (v_cache, 'v_cache')):
-            _require(cache, name, qkv.dtype)
-            if cache.ndim != 4 or tuple(cache.shape[1:]) != (kv_heads, page_size, head_dim):
-                raise ValueError(f'{name} must be [pages, {kv_heads}, {page_size}, {head_dim}]')
+        _check_caches(k_cache, v_cache, dtype, kv_heads, page_size, head_dim)
+    q = torch.empty((n, heads * head_dim), dtype=dtype, device=qkv.device)
     _check(library.load().qil_qk_norm_rope_store(
-        _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots),
-        _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps), _code(qkv.dtype),
-        _stream()), 'qk_norm_rope_store')
+        pointer, code, splits, _ptr(q), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions),
+        _ptr(slots), _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps),
+        _code(dtype), _stream()), 'qk_norm_rope_store')
+    return q
 
 
-def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
+def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window):
     """Attention of every row of the step over its request's cached keys.
 
-    q is read from the leading ``heads * head_dim`` columns of ``qkv`` [N, (heads + 2 kv_heads) d].
-    Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
+    ``q`` [N, heads * head_dim] (head h at columns [h d, (h + 1) d)).  Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
     j <= positions[n] and, with a window, j > positions[n] - window.  -> T [N, heads * head_dim].
 
     Sequences with two or more rows (``cu_seqlens``, ``seq_starts``) go to the matrix-core tile
     kernel; rows alone in their sequence (``single_rows``: their indices, or None when every row is
     alone, i.e. ``max_query == 1``) go to the split-context row kernel.
     """
-    n = qkv.shape[0]
+    n = q.shape[0]
+    qkv = q
     check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=head_dim, dtype=qkv.dtype)
-    _require(qkv, 'qkv', None, (n, (heads + 2 * kv_heads) * head_dim))
+    _require(q, 'q', None, (n, heads * head_dim))
     _require(block_tables, 'block_tables', torch.int32)
     _require(row_seq, 'row_seq', torch.int32, (n,))
     _require(positions, 'positions', torch.int32, (n,))
-    for cache, name in ((k_cache, 'k_cache'), (v_cache, 'v_cache')):
-        _require(cache, name, qkv.dtype)
-        if cache.ndim != 4 or tuple(cache.shape[1:]) != (kv_heads, page_size, head_dim):
-            raise ValueError(f'{name} must be [pages, {kv_heads}, {page_size}, {head_dim}]')
+    _check_caches(k_cache, v_cache, qkv.dtype, kv_heads, page_size, head_dim)
     if block_tables.ndim != 2 or block_tables.shape[1] * page_size < max_context:
         raise ValueError('block_tables are too narrow for the longest context')
     lib = library.load()
@@ -224,14 +267,29 @@ def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_si
     else:
         single_rows, rows = None, n
     if rows:
-        part = ATTENTION_PART
-        parts = max(1, -(-max_context // part))
-        nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
-        workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
-        _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
-                                 block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
-                                 _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
-                                 int(window or 0), float(scale), part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
+        window_arg = int(window or 0)
+        if qkv.dtype == torch.bfloat16 and lib.qil_attn_decode_takes(heads, kv_heads, head_dim, page_size):
+            # matrix-core kernel; split the context until the chip has about four blocks per CU
+            wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
+            part = min(1024, max(64, -(-(-(-max_context // wanted)) // 64) * 64))
+            parts = max(1, -(-max_context // part))
+            nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
+            workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
+            _check(lib.qil_attn_decode(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                       block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
+                                       _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
+                                       window_arg, float(scale), part, parts, _stream()), 'attn_decode')
+            _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), _ptr(single_rows), _ptr(out), rows, heads,
+                                      head_dim, window_arg, part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
+        else:
+            part = ATTENTION_PART
+            parts = max(1, -(-max_context // part))
+            nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
+            workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
+            _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                     block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
+                                     _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
+                                     window_arg, float(scale), part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
     return out
 
 
@@ -245,8 +303,10 @@ def sample(logits, temperatures, seeds, counters):
     _require(temperatures, 'temperatures', torch.float32, (m,))
     _require(seeds, 'seeds', torch.int32, (m,))
     _require(counters, 'counters', torch.int32, (m,))
+    lib = library.load()
     tokens = torch.empty(m, dtype=torch.int32, device=logits.device)
     finite = torch.empty(m, dtype=torch.int32, device=logits.device)
-    _check(library.load().qil_sample(_ptr(logits), _ptr(temperatures), _ptr(seeds), _ptr(counters), _ptr(tokens),
-                                     _ptr(finite), m, vocab, _stream()), 'sample')
+    workspace = torch.empty(lib.qil_sample_workspace(m, vocab) // 4, dtype=torch.int32, device=logits.device)
+    _check(lib.qil_sample(_ptr(logits), _ptr(temperatures), _ptr(seeds), _ptr(counters), _ptr(tokens), _ptr(finite),
+                          _ptr(workspace), m, vocab, _stream()), 'sample')
     return tokens, finite

@@ -138,17 +138,25 @@ def load():
 def _declare(lib):
     p, i, f, z = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
     lib.qil_embed.argtypes = [p, p, p, i, i, i, p]
-    lib.qil_add_rmsnorm.argtypes = [p, p, p, p, p, i, i, f, i, i, p]
-    lib.qil_silu_mul.argtypes = [p, p, i, i, i, p]
+    lib.qil_add_rmsnorm.argtypes = [p, p, i, i, i, p, p, p, i, i, f, i, i, p]
+    lib.qil_silu_mul.argtypes = [p, i, i, p, i, i, i, p]
     lib.qil_add_bias.argtypes = [p, p, i, i, i, p]
-    lib.qil_qk_norm_rope_store.argtypes = [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, p]
+    lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, p]
     lib.qil_attn_rows_workspace.argtypes = [i, i, i, i]
     lib.qil_attn_rows_workspace.restype = z
     lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
+    lib.qil_attn_decode_takes.restype = i
+    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, p]
     lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, p]
-    lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, p]
-    lib.qil_sample.argtypes = [p, p, p, p, p, p, i, i, p]
+    lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, i, p]
+    lib.qil_gemm_bf16_splits.argtypes = [i, i, i]
+    lib.qil_gemm_bf16_splits.restype = i
+    lib.qil_sample.argtypes = [p, p, p, p, p, p, p, i, i, p]
+    lib.qil_sample_workspace.argtypes = [i, i]
+    lib.qil_sample_workspace.restype = z
     for name in ('qil_embed', 'qil_add_rmsnorm', 'qil_silu_mul', 'qil_add_bias', 'qil_qk_norm_rope_store',
-                 'qil_attn_rows', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_sample'):
+                 'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_sample'):
         getattr(lib, name).restype = i

@@ -53,20 +53,20 @@ class Attention(Mixer):
 
     def forward(self, h, ctx, cache):
         p = self.p
-        qkv = ops.linear(h, self.w_qkv, self.b_qkv)
+        qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
-        ops.qk_norm_rope_store(
+        q = ops.qk_norm_rope_store(
             qkv, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
             eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
             rotation=rotation, positions=ctx.positions,
             slots=cache.slots if cache.writes else None,
-            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size)
+            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype)
         attended = ops.paged_attention(
-            qkv, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
+            q, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
             max_query=ctx.max_query, max_context=ctx.max_context,
             scale=self.scale, window=self.window)
-        return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'))
+        return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

@@ -96,6 +96,8 @@ class Rotation:
 class Mixer(Part):
     """Token mixer: [N, width] -> [N, width] over the step's batch and the cache.
 
+    The result is a tensor of the model's type or ``ops.Partials`` (float32 partial sums that the
+    next norm adds).
     ``cache_need()`` says what it keeps between steps (KVNeed, StateNeed or None);
     ``forward(h, ctx, cache)`` gets the step context (engine/batch.py) and the
     cache view of its schedule entry (cache/manager.py: KVView or StateView).
@@ -109,7 +111,7 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Per-token map [N, width] -> [N, width]."""
+    """Per-token map [N, width] -> [N, width] (tensor of the model's type or ``ops.Partials``)."""
     def forward(self, h):
         raise NotImplementedError
 

@@ -10,8 +10,9 @@ class GatedMLP(FeedForward):
     the kernels have.  Gate and up matrices are stacked at ``finalize`` into one
     [2 * intermediate, width] matrix (gate rows first): a pure re-layout."""
 
-    def __init__(self, *, width, intermediate, activation='silu'):
+    def __init__(self, *, width, intermediate, activation='silu', dtype=torch.bfloat16):
         super().__init__()
+        self.dtype = dtype
         if activation != 'silu':
             raise ValueError(f'no kernel for activation {activation!r}')
         self.width, self.intermediate, self.activation = width, intermediate, activation
@@ -26,5 +27,5 @@ class GatedMLP(FeedForward):
         p['gate_up_proj.weight'] = torch.cat([p.pop('gate_proj.weight'), p.pop('up_proj.weight')]).contiguous()
 
     def forward(self, h):
-        gate_up = ops.linear(h, self.p['gate_up_proj.weight'], None)
-        return ops.linear(ops.silu_mul(gate_up), self.p['down_proj.weight'], None)
+        gate_up = ops.linear(h, self.p['gate_up_proj.weight'], None, partials=True)
+        return ops.linear(ops.silu_mul(gate_up, self.dtype), self.p['down_proj.weight'], None, partials=True)

@@ -8,6 +8,11 @@ are test code: the engine never imports them.
 import torch
 
 
+def _value(x):
+    """A tensor, or the sum of float32 partial sums."""
+    return x.sum() if hasattr(x, 'splits') else x
+
+
 def _round(x, dtype):
     return x.to(dtype).to(torch.float32)
 
@@ -23,59 +28,62 @@ def _norm(x, weight, eps, out_dtype):
 
 def add_rmsnorm(stream, delta, weight, eps, out_dtype):
     if delta is not None:
-        stream += delta.to(torch.float32)
+        stream += _value(delta).to(torch.float32)
     return _norm(stream, weight, eps, out_dtype)
 
 
 def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
     x = stream[rows.long()]
     if delta is not None:
-        x = x + delta[rows.long()].to(torch.float32)
+        x = x + _value(delta)[rows.long()].to(torch.float32)
     return _norm(x, weight, eps, out_dtype)
 
 
-def linear(x, weight, bias=None, out_dtype=None):
+def linear(x, weight, bias=None, out_dtype=None, partials=False):
     y = x.to(torch.float32) @ weight.to(torch.float32).t()
     if bias is not None:
         y = y + bias
     return y.to(out_dtype or x.dtype)
 
 
-def silu_mul(gate_up):
+def silu_mul(gate_up, out_dtype=None):
+    gate_up = _value(gate_up)
     inner = gate_up.shape[1] // 2
     g, u = gate_up[:, :inner].to(torch.float32), gate_up[:, inner:].to(torch.float32)
-    return (g / (1 + torch.exp(-g)) * u).to(gate_up.dtype)
+    return (g / (1 + torch.exp(-g)) * u).to(out_dtype or gate_up.dtype)
 
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size):
+                       k_cache, v_cache, page_size, dtype):
+    qkv = _value(qkv)
     n, d = qkv.shape[0], head_dim
     x = qkv.view(n, heads + 2 * kv_heads, d)
     q, k, v = x[:, :heads].to(torch.float32), x[:, heads:heads + kv_heads].to(torch.float32), x[:, heads + kv_heads:]
 
     def shape(t, weight):
         if weight is not None:
-            t = _round(t * torch.rsqrt(t.square().mean(dim=-1, keepdim=True) + eps), qkv.dtype) * weight
+            t = _round(t * torch.rsqrt(t.square().mean(dim=-1, keepdim=True) + eps), dtype) * weight
         if rotation is not None:
             rot, half = rotation.rot_dim, rotation.rot_dim // 2
             c = rotation.cos[positions.long()][:, None, :]
             s = rotation.sin[positions.long()][:, None, :]
             left, right = t[..., :half], t[..., half:rot]
             t = torch.cat((left * c - right * s, left * s + right * c, t[..., rot:]), dim=-1)
-        return t.to(qkv.dtype)
+        return t.to(dtype)
 
-    x[:, :heads] = shape(q, q_weight)
     if slots is not None:
         page, offset = slots.long() // page_size, slots.long() % page_size
         k_cache[page, :, offset] = shape(k, k_weight)
-        v_cache[page, :, offset] = v
+        v_cache[page, :, :, offset] = v.to(dtype)        # V is [pages, kv_heads, d, page_size]
+    return shape(q, q_weight).reshape(n, heads * d)
 
 
-def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
+def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
                     accumulate=torch.float32):
-    n, d, g = qkv.shape[0], head_dim, heads // kv_heads
-    q = qkv[:, :heads * d].reshape(n, heads, d).to(accumulate)
+    n, d, g = q.shape[0], head_dim, heads // kv_heads
+    qkv = q
+    q = q.reshape(n, heads, d).to(accumulate)
     out = torch.empty((n, heads, d), dtype=accumulate, device=qkv.device)
     for row in range(n):
         ctx = int(positions[row]) + 1
@@ -83,7 +91,7 @@ def paged_attention(qkv, *, heads, kv_heads, head_dim, k_cache, v_cache, page_si
         j = torch.arange(lo, ctx, device=qkv.device)
         pages = block_tables[int(row_seq[row])].long()[j // page_size]
         keys = k_cache[pages, :, j % page_size].to(accumulate)          # [ctx, kv_heads, d]
-        values = v_cache[pages, :, j % page_size].to(accumulate)
+        values = v_cache[pages, :, :, j % page_size].to(accumulate)     # [ctx, kv_heads, d]
         keys = keys.repeat_interleave(g, dim=1)
         values = values.repeat_interleave(g, dim=1)
         scores = torch.einsum('hd,jhd->hj', q[row], keys) * scale

@@ -64,6 +64,25 @@ def test_add_rmsnorm(ops, dtype, rows, width):
     check(got, refs.rows_rmsnorm(stream, delta, rows_index, weight, 1e-5, dtype), dtype, scale=4)
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('rows,width,splits', [(3, 72, 1), (8, 4096, 4), (5, 1000, 2), (2, 6000, 3)])
+def test_add_rmsnorm_of_partial_sums(ops, dtype, rows, width, splits):
+    """The delta as float32 partial sums of a K-split product: added in split order."""
+    stream = rand(rows, width, scale=3.0)
+    parts = rand(splits, rows, width, seed=5)
+    weight = (1 + 0.3 * rand(width, seed=2)).contiguous()
+    want_stream = stream.clone()
+    for i in range(splits):                       # the kernel's order: stream + p0 + p1 + ...
+        want_stream += parts[i]
+    want = refs.add_rmsnorm(want_stream.clone(), None, weight, 1e-6, dtype)
+    got_stream = stream.clone()
+    got = ops.add_rmsnorm(got_stream, ops.Partials(parts), weight, 1e-6, dtype)
+    torch.testing.assert_close(got_stream, want_stream, atol=1e-6, rtol=1e-6)
+    check(got, want, dtype, scale=4)
+    index = torch.tensor([rows - 1], dtype=torch.int32).cuda()
+    check(ops.rows_rmsnorm(stream, ops.Partials(parts), index, weight, 1e-6, dtype), want[rows - 1:], dtype, scale=4)
+
+
 def test_rmsnorm_rounds_before_the_weight(ops):
     """bfloat16: the normalised value is rounded, then multiplied by the weight (qil/model.py:22-23)."""
     width = 64
@@ -103,6 +122,18 @@ def test_linear_bfloat16(ops, m, n, k, out_dtype, bias):
         check(got, want, torch.bfloat16, scale=2)
 
 
+@pytest.mark.parametrize('m,n,k', [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 12288), (64, 1024, 3072), (16, 130, 52),
+                                   (3, 96, 224), (40, 200, 1030)])
+def test_linear_partial_sums(ops, m, n, k):
+    """Few rows, bfloat16: the product may come back split over K; the parts add up to it."""
+    x, w = rand(m, k, dtype=torch.bfloat16), rand(n, k, dtype=torch.bfloat16, seed=1, scale=k ** -0.5)
+    got = ops.linear(x, w, None, partials=True)
+    assert isinstance(got, ops.Partials) and got.shape == (m, n)
+    check(got.sum(), x.double() @ w.double().t(), torch.float32, scale=8)
+    if k >= 4096 and n <= 8192:
+        assert got.splits > 1, 'a product with few columns and a long K should be split'
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops):
     """A row's result is the same alone, among 7 and among 40 (same kernel family): bit for bit."""
     x, w = rand(40, 512, dtype=torch.bfloat16), rand(300, 512, dtype=torch.bfloat16, seed=1, scale=0.05)
@@ -116,6 +147,10 @@ def test_silu_mul(ops, dtype):
     gate_up = rand(7, 2 * 136, dtype=dtype, scale=3.0)
     want = torch.nn.functional.silu(gate_up[:, :136].double()) * gate_up[:, 136:].double()
     check(ops.silu_mul(gate_up), want, dtype, scale=8)
+    parts = rand(3, 7, 2 * 136, scale=2.0, seed=9)
+    total = parts[0] + parts[1] + parts[2]
+    want = torch.nn.functional.silu(total[:, :136].double()) * total[:, 136:].double()
+    check(ops.silu_mul(ops.Partials(parts), dtype), want, dtype, scale=8)
 
 
 class Rot:
@@ -135,26 +170,30 @@ def test_qk_norm_rope_store(ops, dtype, heads, kv_heads, d, rot, page_size):
     rotation = Rot(d, 10000.0, 600, rot)
     positions = torch.tensor([0, 1, 2, 17, 18, 19, 500, 3, 599], dtype=torch.int32).cuda()
     slots = torch.randperm(pages * page_size)[:n].to(torch.int32).cuda()
-    caches = [torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype).cuda() for _ in range(4)]
+    caches = [torch.full((pages, kv_heads, page_size, d) if i % 2 == 0 else (pages, kv_heads, d, page_size), float('nan'),
+                         dtype=dtype).cuda() for i in range(4)]
     args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, q_weight=qw, k_weight=kw, eps=1e-5, rotation=rotation,
-                positions=positions, slots=slots, page_size=page_size)
-    want = qkv.clone()
-    refs.qk_norm_rope_store(want, k_cache=caches[0], v_cache=caches[1], **args)
-    got = qkv.clone()
-    ops.qk_norm_rope_store(got, k_cache=caches[2], v_cache=caches[3], **args)
-    q = heads * d
-    check(got[:, :q], want[:, :q], dtype, scale=4)
+                positions=positions, slots=slots, page_size=page_size, dtype=dtype)
+    want = refs.qk_norm_rope_store(qkv.clone(), k_cache=caches[0], v_cache=caches[1], **args)
+    got = ops.qk_norm_rope_store(qkv.clone(), k_cache=caches[2], v_cache=caches[3], **args)
+    check(got, want, dtype, scale=4)
     for mine, theirs in ((caches[2], caches[0]), (caches[3], caches[1])):
         written = ~torch.isnan(theirs.float())
         assert (written == ~torch.isnan(mine.float())).all(), 'other slots were written'
         check(mine[written], theirs[written], dtype, scale=4)
     # a reader of another entry's cache stores nothing and still shapes q
     untouched = [c.clone() for c in caches[2:]]
-    again = qkv.clone()
-    ops.qk_norm_rope_store(again, k_cache=caches[2], v_cache=caches[3], **{**args, 'slots': None})
-    torch.testing.assert_close(again[:, :q], got[:, :q], atol=0, rtol=0)
+    again = ops.qk_norm_rope_store(qkv.clone(), k_cache=caches[2], v_cache=caches[3], **{**args, 'slots': None})
+    torch.testing.assert_close(again, got, atol=0, rtol=0)
     for before, after in zip(untouched, caches[2:]):
         assert torch.equal(torch.nan_to_num(before.float()), torch.nan_to_num(after.float()))
+    # the same from float32 partial sums
+    halves = torch.stack((qkv.float() * 0.25, qkv.float() * 0.75)).contiguous()
+    fresh = [torch.full_like(c, float('nan')) for c in caches[2:]]
+    split = ops.qk_norm_rope_store(ops.Partials(halves), k_cache=fresh[0], v_cache=fresh[1], **args)
+    check(split, want, dtype, scale=4)
+    written = ~torch.isnan(caches[0].float())
+    check(fresh[0][written], caches[0][written], dtype, scale=4)
 
 
 def test_rotation_pairs_and_signs(ops):
@@ -165,13 +204,14 @@ def test_rotation_pairs_and_signs(ops):
     qkv[0, 0] = 1.0
     rotation = Rot(d, 1.0, 8)              # theta 1: every frequency is 1, angle = position
     cache = torch.zeros(1, 1, 4, d).cuda()
-    ops.qk_norm_rope_store(qkv, heads=1, kv_heads=1, head_dim=d, q_weight=None, k_weight=None, eps=0.0,
-                           rotation=rotation, positions=torch.tensor([p], dtype=torch.int32).cuda(),
-                           slots=torch.tensor([2], dtype=torch.int32).cuda(), k_cache=cache, v_cache=cache.clone(),
-                           page_size=4)
+    v_cache = torch.zeros(1, 1, d, 4).cuda()
+    q = ops.qk_norm_rope_store(qkv, heads=1, kv_heads=1, head_dim=d, q_weight=None, k_weight=None, eps=0.0,
+                               rotation=rotation, positions=torch.tensor([p], dtype=torch.int32).cuda(),
+                               slots=torch.tensor([2], dtype=torch.int32).cuda(), k_cache=cache, v_cache=v_cache,
+                               page_size=4, dtype=torch.float32)
     expected = torch.zeros(d)
     expected[0], expected[d // 2] = torch.cos(torch.tensor(3.0)), torch.sin(torch.tensor(3.0))
-    torch.testing.assert_close(qkv[0, :d].cpu(), expected, atol=1e-6, rtol=0)
+    torch.testing.assert_close(q[0].cpu(), expected, atol=1e-6, rtol=0)
 
 
 def build_cache(lengths, page_size, kv_heads, d, dtype, seed=37):
@@ -179,7 +219,7 @@ def build_cache(lengths, page_size, kv_heads, d, dtype, seed=37):
     torch.manual_seed(seed)
     pages = sum(-(-n // page_size) for n in lengths) + 2
     k_cache = torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype)
-    v_cache = torch.full((pages, kv_heads, page_size, d), float('nan'), dtype=dtype)
+    v_cache = torch.full((pages, kv_heads, d, page_size), float('nan'), dtype=dtype)    # transposed pages
     free, tables = list(range(pages)), [[] for _ in lengths]
     for end in range(1, max(lengths) + page_size, page_size):
         for i, n in enumerate(lengths):
@@ -191,7 +231,7 @@ def build_cache(lengths, page_size, kv_heads, d, dtype, seed=37):
         j = torch.arange(n)
         page = torch.tensor(tables[i])[j // page_size]
         k_cache[page, :, j % page_size] = k
-        v_cache[page, :, j % page_size] = v
+        v_cache[page, :, :, j % page_size] = v
         histories.append((k, v))
     width = max(len(t) for t in tables)
     table = torch.tensor([t + [0] * (width - len(t)) for t in tables], dtype=torch.int32)
@@ -215,7 +255,7 @@ ATT_TOL = {torch.float32: dict(atol=2e-6, rtol=2e-5), torch.bfloat16: dict(atol=
 def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, kv_heads):
     k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
     rows = len(lengths)
-    qkv = rand(rows, (heads + 2 * kv_heads) * d, dtype=dtype)
+    qkv = rand(rows, heads * d, dtype=dtype)
     positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
     row_seq = torch.arange(rows, dtype=torch.int32).cuda()
     args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
@@ -224,7 +264,7 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
     got = ops.paged_attention(qkv, **args)
     expected = []
     for row, (k, v) in enumerate(histories):             # float64, explicit GQA map (:35-40)
-        q = qkv[row, :heads * d].reshape(heads, d).double().cpu()
+        q = qkv[row].reshape(heads, d).double().cpu()
         kh = k.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
         vh = v.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
         score = (q[:, None, :] * kh).sum(-1) * d ** -0.5
@@ -236,7 +276,7 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
         j = torch.arange(lengths[1])
         page = table[1].long()[j // page_size]
         k_cache[page, :, j % page_size] = 999.0
-        v_cache[page, :, j % page_size] = -999.0
+        v_cache[page, :, :, j % page_size] = -999.0
         torch.testing.assert_close(ops.paged_attention(qkv, **args)[0], got[0], atol=0, rtol=0)
 
 
@@ -252,13 +292,13 @@ def mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_he
     single = [cu[i] for i, c in enumerate(chunks) if c == 1]
     n = cu[-1]
     dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
-    qkv = rand(n, (heads + 2 * kv_heads) * d, dtype=dtype)
+    qkv = rand(n, heads * d, dtype=dtype)
     got = ops.paged_attention(qkv, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
                               page_size=page_size, block_tables=table, row_seq=dev(row_seq), positions=dev(positions),
                               cu_seqlens=dev(cu), seq_starts=dev(starts), single_rows=dev(single) if max(chunks) > 1 else None,
                               n_seqs=len(lengths), max_query=max(chunks), max_context=max(lengths), scale=scale,
                               window=window)
-    q = qkv[:, :heads * d].reshape(n, heads, d).double().cpu()
+    q = qkv.reshape(n, heads, d).double().cpu()
     expected = torch.cat([
         plain.attention(q[cu[i]:cu[i + 1]], histories[i][0].double(), histories[i][1].double(),
                         torch.arange(starts[i], lengths[i]), scale, window)
@@ -295,7 +335,7 @@ def test_one_far_key_among_hundreds(ops):
     page_size, d, heads, kv_heads, n = 16, 64, 8, 2, 900
     k_cache, v_cache, table, histories = build_cache([n], page_size, kv_heads, d, torch.float32)
     target = 37
-    q = rand(1, (heads + 2 * kv_heads) * d)
+    q = rand(1, heads * d)
     for h in range(heads):
         kvh = h // (heads // kv_heads)
         direction = histories[0][0][target, kvh] / histories[0][0][target, kvh].norm()
