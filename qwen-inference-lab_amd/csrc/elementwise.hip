@@ -12,14 +12,6 @@ __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
 }
 
-// A sub-layer's output arrives either in the model's type T (one array) or as float32 partial sums
-// of a K-split matrix product, [splits][rows][width], which the consumer adds in split order.
-template <typename TD>
-__device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t index, int splits, size_t stride) {
-  float v = ld(base + index);
-  for (int s = 1; s < splits; ++s) v += ld(base + s * stride + index);
-  return v;
-}
 __device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ float4 load4(const bf16_t* p) {
   const uint2 raw = *reinterpret_cast<const uint2*>(p);
@@ -32,6 +24,34 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
                                             (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16));
 }
 
+// A sub-layer's output arrives either in the model's type T (one array) or as float32 partial sums
+// of a K-split matrix product, [splits][rows][width], which the consumer adds in split order.
+// Loads go out eight at a time before the first is used; the additions stay in split order.
+template <typename TD>
+__device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t index, int splits, size_t stride) {
+  float v = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = s0 + u < splits ? ld(base + (s0 + u) * stride + index) : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v += part[u];
+  }
+  return v;
+}
+template <typename TD>
+__device__ __forceinline__ float4 load_sum4(const TD* __restrict__ base, size_t index, int splits, size_t stride) {
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float4 part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      part[u] = s0 + u < splits ? load4(base + (s0 + u) * stride + index) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { v.x += part[u].x; v.y += part[u].y; v.z += part[u].z; v.w += part[u].w; }
+  }
+  return v;
+}
 // One block per output row.
 //   x = stream[r] (+ delta[r]);  if (update) stream[r] = x;
 //   out[m] = round_T(round_T(x * rsqrt(mean(x^2) + eps)) * weight)   (qil/model.py:15-23)
@@ -64,9 +84,10 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ stream, const TD* __restr
   }
 }
 
-// The same for width % 4 == 0 and width <= 16 * THREADS: the row stays in registers between the
-// two passes and every access is a 16-byte (8-byte for bfloat16) vector.
-template <typename TD, typename T, int THREADS>
+// The same for width % 4 == 0 and width <= 4 * J * THREADS: every access is a 16-byte (8-byte for
+// bfloat16) vector, all loads (stream, delta or its partial sums, weight) are issued before the first
+// is used, and the row stays in registers between the statistics and the output.
+template <typename TD, typename T, int THREADS, int J>
 __global__ void __launch_bounds__(THREADS)
 add_rmsnorm_vec_kernel(float* __restrict__ stream, const TD* __restrict__ delta, int splits, size_t split_stride,
                        const int* __restrict__ rows, const float* __restrict__ weight, T* __restrict__ out, int width,
@@ -75,34 +96,35 @@ add_rmsnorm_vec_kernel(float* __restrict__ stream, const TD* __restrict__ delta,
   const int m = blockIdx.x;
   const size_t r = rows ? (size_t)rows[m] : (size_t)m;
   float* x = stream + r * width;
-  float4 cache[4];
+  float4 cache[J], w[J], d[J];
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    const int i = (threadIdx.x + j * THREADS) * 4;
+    const bool live = i < width;
+    cache[j] = live ? load4(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    w[j] = live ? load4(weight + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    d[j] = (live && delta) ? load_sum4(delta, r * width + i, splits, split_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
   float sum = 0.f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < J; ++j) {
     const int i = (threadIdx.x + j * THREADS) * 4;
-    if (i < width) {
-      float4 v = load4(x + i);
-      if (delta) {
-        for (int s = 0; s < splits; ++s) {
-          const float4 d = load4(delta + s * split_stride + r * width + i);
-          v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
-        }
-        if (update) store4(x + i, v);
-      }
-      cache[j] = v;
-      sum += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-    }
+    float4 v = cache[j];
+    v.x += d[j].x; v.y += d[j].y; v.z += d[j].z; v.w += d[j].w;
+    if (delta && update && i < width) store4(x + i, v);
+    cache[j] = v;
+    sum += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
   }
   sum = block_sum(sum, scratch);
   const float rstd = rsqrtf(sum / (float)width + eps);
   T* y = out + (size_t)m * width;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < J; ++j) {
     const int i = (threadIdx.x + j * THREADS) * 4;
     if (i < width) {
-      const float4 v = cache[j], w = load4(weight + i);
-      store4(y + i, make_float4(round_to<T>(v.x * rstd) * w.x, round_to<T>(v.y * rstd) * w.y,
-                                round_to<T>(v.z * rstd) * w.z, round_to<T>(v.w * rstd) * w.w));
+      const float4 v = cache[j];
+      store4(y + i, make_float4(round_to<T>(v.x * rstd) * w[j].x, round_to<T>(v.y * rstd) * w[j].y,
+                                round_to<T>(v.z * rstd) * w[j].z, round_to<T>(v.w * rstd) * w[j].w));
     }
   }
 }
@@ -148,16 +170,17 @@ int qil_add_rmsnorm(float* stream, const void* delta, int delta_dtype, int split
   if (n_out == 0) return 0;
   if (splits < 1 || (delta_dtype == QIL_BF16 && splits != 1)) return -1;
   const size_t stride = (size_t)delta_rows * width;
-  const bool vec = width % 4 == 0 && width <= 16 * 256 &&
+  const bool vec = width % 4 == 0 && width <= 8192 &&
                    (((uintptr_t)stream | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) % 16 == 0);
+#define QIL_NORM_VEC(TD, T, THREADS, J)                                                                             \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, T, THREADS, J>), dim3(n_out), dim3(THREADS), 0, s, stream,          \
+                     (const TD*)delta, splits, stride, rows, weight, (T*)out, width, eps, update)
 #define QIL_NORM_CASE(TD, T)                                                                                         \
   do {                                                                                                               \
-    if (vec && width <= 16 * 64)                                                                                     \
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, T, 64>), dim3(n_out), dim3(64), 0, s, stream, (const TD*)delta, \
-                         splits, stride, rows, weight, (T*)out, width, eps, update);                                 \
-    else if (vec)                                                                                                    \
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, T, 256>), dim3(n_out), dim3(256), 0, s, stream,                 \
-                         (const TD*)delta, splits, stride, rows, weight, (T*)out, width, eps, update);               \
+    if (vec && width <= 256) QIL_NORM_VEC(TD, T, 64, 1);                                                             \
+    else if (vec && width <= 1024) QIL_NORM_VEC(TD, T, 256, 1);                                                      \
+    else if (vec && width <= 4096) QIL_NORM_VEC(TD, T, 1024, 1);                                                     \
+    else if (vec) QIL_NORM_VEC(TD, T, 1024, 2);                                                                      \
     else                                                                                                             \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, T>), dim3(n_out), dim3(width >= 2048 ? 512 : width >= 512 ? 256 : 64), \
                          0, s, stream, (const TD*)delta, splits, stride, rows, weight, (T*)out, width, eps, update); \
@@ -171,6 +194,7 @@ int qil_add_rmsnorm(float* stream, const void* delta, int delta_dtype, int split
     QIL_NORM_CASE(bf16_t, bf16_t);
   }
 #undef QIL_NORM_CASE
+#undef QIL_NORM_VEC
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -1,16 +1,16 @@
 // bfloat16 matrix product on the matrix cores for few rows (decode, selected logit rows):
 //   C[M, N] = A[M, K] W[N, K]^T (+ bias[N]),  float32 accumulation.
 // Both operands have K contiguous (qil/model.py:32-40).  The product is bound by streaming W once
-// from HBM, so the kernel is shaped to keep as many loads in flight as the chip can hold:
+// from HBM; A is small and would be re-read from L2 by every block, so the work is cut into wide,
+// short pieces: a block owns 128 * NT rows of W (8 waves, each 16 * NT rows) and ONE of `splits`
+// ranges of K.  It stages its slice of A in LDS once, then every wave streams its rows of W from
+// global memory straight into v_mfma_f32_16x16x32_bf16 operands, loading UNROLL k steps ahead of
+// the first product that uses them.  A's traffic is M / (128 NT) of W's.
 //
-//   * a block owns 16 rows of W (16 output columns), 16 * MT rows of A and one of `splits` ranges
-//     of K; its waves split that range into contiguous pieces, and every wave issues the loads
-//     of four 32-wide k steps before the first v_mfma_f32_16x16x32_bf16 that uses them;
-//   * with few columns (N / 16 blocks would leave CUs idle) K is split over blocks as well:
-//     the block writes a float32 partial result C[split, M, N], and the kernel that consumes
-//     the product (norm, rotary/store, SiLU gate) adds the partials in split order.  Sums are
-//     therefore made in a fixed order: the waves' in wave order, the splits' in split order;
-//   * with splits == 1 the result may be rounded to bfloat16 here (and take the bias).
+// With splits > 1 a block writes a float32 partial result C[split, M, N], and the kernel that
+// consumes the product (norm, rotary/store, SiLU gate) adds the partials in split order, so
+// every sum is made in a fixed order.  With splits == 1 the result may be rounded to bfloat16
+// here and take the bias.
 //
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (wave64): lane l supplies A[l % 16][8 (l / 16) .. +7]
 // and B[8 (l / 16) .. +7][l % 16]; it receives D[4 (l / 16) + i][l % 16], i < 4.  A and W rows are
@@ -42,111 +42,147 @@ __device__ __forceinline__ uint4 load_frag(const bf16_t* __restrict__ base, int 
   return raw;
 }
 
-#define GEMM_UNROLL 4
+#define GEMM_WAVES 8
+#define GEMM_LDS_PAD 8          // bf16 elements between rows of the staged A slice
 
-template <int MT, int WAVES, bool ALIGNED, typename OUT>
-__global__ void __launch_bounds__(WAVES * QIL_WAVE)
+// chunk: k columns of A staged at a time (a multiple of 32); the block's range is walked in chunks.
+template <int MT, int NT, int UNROLL, bool ALIGNED, typename OUT>
+__global__ void __launch_bounds__(GEMM_WAVES * QIL_WAVE)
 gemm_bf16_stream_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-                        OUT* __restrict__ C, int M, int N, int K, int steps_per_split) {
-  __shared__ float partial[WAVES][MT][256];
+                        OUT* __restrict__ C, int M, int N, int K, int steps_per_split, int chunk) {
+  extern __shared__ __align__(16) bf16_t a_lds[];          // [16 MT][chunk + pad]
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16 * MT, split = blockIdx.z;
+  const int n0 = (blockIdx.x * GEMM_WAVES + wave) * 16 * NT, m0 = blockIdx.y * 16 * MT, split = blockIdx.z;
+  const int row_width = chunk + GEMM_LDS_PAD;
 
-  f32x4 acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  // this block's k steps, cut into contiguous pieces for the waves
-  const int steps = (K + 31) / 32;
-  const int s0 = split * steps_per_split, s1 = min(steps, s0 + steps_per_split);
-  const int per_wave = (s1 - s0 + WAVES - 1) / WAVES;
-  const int w0 = s0 + wave * per_wave, w1 = min(s1, w0 + per_wave);
-  for (int step = w0; step < w1; step += GEMM_UNROLL) {
-    uint4 b[GEMM_UNROLL], a[GEMM_UNROLL][MT];
-#pragma unroll
-    for (int u = 0; u < GEMM_UNROLL; ++u) {
-      const int k = (step + u < w1) ? (step + u) * 32 + kb * 8 : K;      // K: out of range, loads nothing
-      b[u] = load_frag<ALIGNED>(W, n0 + r, N, k, K);
-#pragma unroll
-      for (int t = 0; t < MT; ++t) a[u][t] = load_frag<ALIGNED>(A, m0 + t * 16 + r, M, k, K);
-    }
-#pragma unroll
-    for (int u = 0; u < GEMM_UNROLL; ++u)
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u][t]),
-                                                         __builtin_bit_cast(bf16x8, b[u]), acc[t], 0, 0, 0);
-  }
-  // lane holds D[4 kb + i][r]; park it as [m][n] so the final pass is contiguous in n
+  f32x4 acc[MT][NT];
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) partial[wave][t][(4 * kb + i) * 16 + r] = acc[t][i];
-  __syncthreads();
-  OUT* out = C + (size_t)split * M * N;
-  for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * QIL_WAVE) {
-    const int t = idx >> 8, cell = idx & 255;
-    const int m = m0 + t * 16 + (cell >> 4), n = n0 + (cell & 15);
-    if (m >= M || n >= N) continue;
-    float total = 0.f;
+    for (int j = 0; j < NT; ++j) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int k_begin = split * steps_per_split * 32, k_end = min(K, k_begin + steps_per_split * 32);
+  for (int kc = k_begin; kc < k_end; kc += chunk) {
+    const int width = min(chunk, k_end - kc);               // columns of this chunk (last one may be short)
+    __syncthreads();                                        // the previous chunk is consumed
+    for (int idx = threadIdx.x; idx < 16 * MT * (chunk / 8); idx += GEMM_WAVES * QIL_WAVE) {
+      const int m = idx / (chunk / 8), c = (idx - m * (chunk / 8)) * 8;
+      const uint4 v = c < width ? load_frag<ALIGNED>(A, m0 + m, M, kc + c, K) : make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+    }
+    __syncthreads();
+    const int steps = (width + 31) / 32;
+    for (int step = 0; step < steps; step += UNROLL) {
+      uint4 b[UNROLL][NT];
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) total += partial[w][t][cell];
-    store_out(out + (size_t)m * N + n, total + (bias ? bias[n] : 0.f));
+      for (int u = 0; u < UNROLL; ++u) {
+        const int k = (step + u < steps) ? kc + (step + u) * 32 + kb * 8 : K;    // K: out of range, loads nothing
+#pragma unroll
+        for (int j = 0; j < NT; ++j) b[u][j] = load_frag<ALIGNED>(W, n0 + j * 16 + r, N, k, K);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (step + u < steps) {
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const uint4 a = *reinterpret_cast<const uint4*>(a_lds + (t * 16 + r) * row_width + (step + u) * 32 + kb * 8);
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+              acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                  __builtin_bit_cast(bf16x8, b[u][j]), acc[t][j], 0, 0, 0);
+          }
+        }
+      }
+    }
   }
+  // lane holds D[m = 4 kb + i][n = r] of each tile
+  OUT* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + t * 16 + 4 * kb + i, n = n0 + j * 16 + r;
+        if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[t][j][i] + (bias ? bias[n] : 0.f));
+      }
 }
 
-template <int MT, int WAVES, typename OUT>
-static void launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OUT* C, int M, int N, int K, int splits,
-                          hipStream_t s) {
+template <int MT, int NT, int UNROLL, typename OUT>
+static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OUT* C, int M, int N, int K, int splits,
+                         int chunk, hipStream_t s) {
   const int steps = (K + 31) / 32;
   const int steps_per_split = (steps + splits - 1) / splits;
-  dim3 grid((N + 15) / 16, (M + 16 * MT - 1) / (16 * MT), splits);
+  if (chunk <= 0 || chunk > steps_per_split * 32) chunk = steps_per_split * 32;
+  const size_t cap = 64 * 1024 / (16 * MT * sizeof(bf16_t));             // elements per row that fit 64 KB
+  if ((size_t)chunk + GEMM_LDS_PAD > cap) chunk = (int)((cap - GEMM_LDS_PAD) / 32 * 32);
+  const size_t lds = (size_t)16 * MT * (chunk + GEMM_LDS_PAD) * sizeof(bf16_t);
+  dim3 grid((N + 128 * NT - 1) / (128 * NT), (M + 16 * MT - 1) / (16 * MT), splits);
   const bool aligned = (K % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
   if (aligned)
-    hipLaunchKernelGGL((gemm_bf16_stream_kernel<MT, WAVES, true, OUT>), grid, dim3(WAVES * QIL_WAVE), 0, s, A, W, bias,
-                       C, M, N, K, steps_per_split);
+    hipLaunchKernelGGL((gemm_bf16_stream_kernel<MT, NT, UNROLL, true, OUT>), grid, dim3(GEMM_WAVES * QIL_WAVE), lds, s,
+                       A, W, bias, C, M, N, K, steps_per_split, chunk);
   else
-    hipLaunchKernelGGL((gemm_bf16_stream_kernel<MT, WAVES, false, OUT>), grid, dim3(WAVES * QIL_WAVE), 0, s, A, W, bias,
-                       C, M, N, K, steps_per_split);
+    hipLaunchKernelGGL((gemm_bf16_stream_kernel<MT, NT, UNROLL, false, OUT>), grid, dim3(GEMM_WAVES * QIL_WAVE), lds, s,
+                       A, W, bias, C, M, N, K, steps_per_split, chunk);
+  return 0;
 }
+
+// Shapes of the kernel that exist: code = MT * 100 + NT * 10 + UNROLL.
+#define QIL_GEMM_SHAPES(X) \
+  X(1, 1, 4) X(1, 1, 8) X(1, 2, 4) X(1, 2, 8) X(1, 4, 4) X(2, 1, 4) X(2, 1, 8) X(2, 2, 4) X(4, 1, 4) X(4, 1, 8) \
+  X(4, 2, 4) X(4, 2, 2)
 
 template <typename OUT>
-static void dispatch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OUT* C, int M, int N, int K,
-                            int splits, hipStream_t s) {
-  // Row tiles: 16, 32 or 64 rows of A per pass over W.  Waves per block: as many as have at least
-  // one unrolled group of k steps each.
-  const int steps = ((K + 31) / 32 + splits - 1) / splits;
-  const int waves = steps >= 8 * GEMM_UNROLL ? 8 : steps >= 4 * GEMM_UNROLL ? 4 : 2;
-#define QIL_STREAM_CASE(MT)                                                              \
-  if (waves == 8) launch_stream<MT, 8, OUT>(A, W, bias, C, M, N, K, splits, s);          \
-  else if (waves == 4) launch_stream<MT, 4, OUT>(A, W, bias, C, M, N, K, splits, s);     \
-  else launch_stream<MT, 2, OUT>(A, W, bias, C, M, N, K, splits, s)
-  if (M <= 16) { QIL_STREAM_CASE(1); }
-  else if (M <= 32) { QIL_STREAM_CASE(2); }
-  else { QIL_STREAM_CASE(4); }
-#undef QIL_STREAM_CASE
+static int launch_shape(int code, const bf16_t* A, const bf16_t* W, const float* bias, OUT* C, int M, int N, int K,
+                        int splits, int chunk, hipStream_t s) {
+#define X(MT, NT, UNROLL) \
+  if (code == MT * 100 + NT * 10 + UNROLL) return launch_stream<MT, NT, UNROLL, OUT>(A, W, bias, C, M, N, K, splits, chunk, s);
+  QIL_GEMM_SHAPES(X)
+#undef X
+  return -1;
 }
 
-// How many ways to split K so that the launch has enough waves for the chip, given the columns.
-extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
-  const int tiles = ((N + 15) / 16) * ((M + 63) / 64);
+// The plan for a product: kernel shape code and the number of K splits.
+static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
   const int steps = (K + 31) / 32;
-  int splits = 1;
-  // aim at >= 1024 blocks; keep at least 8 k steps (256 columns of K) per split
-  while (tiles * splits < 1024 && splits < 16 && steps / (splits * 2) >= 8) splits *= 2;
+  const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  const int column_blocks = (N + 127) / 128;
+  int sp = 1;
+  if (may_split) {
+    // about three blocks per CU (256 CUs), at least 8 k steps per split, fewer splits for more rows
+    const int most = 8;                                   // the consumer reads every partial
+    sp = (768 + column_blocks - 1) / column_blocks;
+    if (sp > most) sp = most;
+    while (sp > 1 && steps / sp < 8) --sp;
+    if (sp < 1) sp = 1;
+  }
+  *code = mt * 100 + 10 + 4;
+  *splits = sp;
+}
+
+// How many ways the product will be split over K when partial sums are allowed.
+extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
+  int code, splits;
+  plan(M, N, K, true, &code, &splits);
   return splits;
 }
 
 // out_dtype QIL_BF16: C bfloat16 [M, N], splits must be 1.  QIL_F32: C float32 [splits, M, N], the
 // value being the sum over the first axis; bias (if any) requires splits == 1.
+// shape: 0 = chosen here, else a code of QIL_GEMM_SHAPES; chunk: 0 = chosen here (tuning runs set both).
 extern "C" int qil_gemm_bf16(const void* A, const void* W, const float* bias, void* C, int M, int N, int K,
-                             int out_dtype, int splits, hipStream_t s) {
+                             int out_dtype, int splits, int shape, int chunk, hipStream_t s) {
   if (M == 0 || N == 0) return 0;
   if (K < 1 || splits < 1 || splits > 65535 || (splits > 1 && (out_dtype != QIL_F32 || bias))) return -1;
+  int code = shape, planned;
+  if (!code) plan(M, N, K, false, &code, &planned);
+  int status;
   if (out_dtype == QIL_F32)
-    dispatch_stream<float>((const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, splits, s);
+    status = launch_shape<float>(code, (const bf16_t*)A, (const bf16_t*)W, bias, (float*)C, M, N, K, splits, chunk, s);
   else
-    dispatch_stream<bf16_t>((const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, splits, s);
+    status = launch_shape<bf16_t>(code, (const bf16_t*)A, (const bf16_t*)W, bias, (bf16_t*)C, M, N, K, splits, chunk, s);
+  if (status) return status;
   QIL_RETURN_LAUNCH_STATUS();
 }

@@ -17,10 +17,17 @@
 
 #define QIL_MAX_HEAD_DIM 512
 
+// Loads go out eight at a time before the first is used; the additions stay in split order.
 template <typename TD>
 __device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t index, int splits, size_t stride) {
-  float v = ld(base + index);
-  for (int s = 1; s < splits; ++s) v += ld(base + s * stride + index);
+  float v = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = s0 + u < splits ? ld(base + (s0 + u) * stride + index) : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v += part[u];
+  }
   return v;
 }
 

@@ -15,8 +15,8 @@ import torch
 
 from . import library
 
-# Rows up to which a bfloat16 product runs on the weight-streaming kernel whatever its output type.
-STREAM_GEMM_MAX_ROWS = 64
+# Rows up to which a bfloat16 product runs on the weight-streaming kernel (float32 results: always).
+STREAM_GEMM_MAX_ROWS = 16
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
 # Blocks the matrix-core decode kernel aims for (256 CUs).
@@ -167,11 +167,11 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     if n <= STREAM_GEMM_MAX_ROWS and partials and bias is None and out_dtype == x.dtype:
         splits = lib.qil_gemm_bf16_splits(n, o, k)
         out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
-        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, _stream()), 'gemm_bf16')
+        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, 0, 0, _stream()), 'gemm_bf16')
         return Partials(out)
     if out_dtype == torch.float32 or n <= STREAM_GEMM_MAX_ROWS:
         out = torch.empty((n, o), dtype=out_dtype, device=x.device)
-        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), 1,
+        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), 1, 0, 0,
                                  _stream()), 'gemm_bf16')
         return out
     out = torch.mm(x, weight.t())                      # GPU BLAS, float32 accumulation
