@@ -1,0 +1,101 @@
+"""HIP graphs for decode steps.
+
+A decode step launches some ten small kernels per layer; launched one by one from Python the
+host, not the GPU, sets the pace.  A batch in which every request brings exactly one token and
+wants its logits has the same kernels, grids and tensor shapes whenever the batch size and the
+*bucket* of the longest context are the same, so its launches are captured once into a HIP graph
+and replayed.  What changes from step to step (tokens, positions, block tables, slots) lives in
+one static int32 device array that is overwritten before each replay; kernels read positions
+from it and leave early past a row's context, so one graph serves every context up to the
+bucket's end.
+
+Nothing in the captured region clears memory with a memset node: buffers are allocated, not
+zeroed, and kernels write every element they later read.
+"""
+import gc
+import weakref
+
+import torch
+
+from .batch import StepEntry
+
+BUCKET = 512          # contexts are rounded up to a multiple of this many tokens for a graph
+MAX_GRAPHS = 12
+
+
+class _Graph:
+    def __init__(self, runner, entries, pieces, facts, bucket):
+        self.sizes = [len(p) for p in pieces]
+        total = sum(self.sizes)
+        device = runner.model.device
+        self.meta = torch.zeros(total, dtype=torch.int32, device=device)
+        self.staging = torch.zeros(total, dtype=torch.int32).pin_memory()
+        self.copied = torch.cuda.Event()
+        self.load(pieces)
+        ctx = runner._context(entries, pieces, facts, self.meta, max_context=bucket)
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side):                       # eager once: loads the library, sizes the allocator
+            runner.model.forward(ctx, runner.views)
+        torch.cuda.current_stream(device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        # No garbage collection while capturing: a collected object that frees device or pinned memory
+        # (an older graph, say) would issue a call the capture forbids, and the process would abort.
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = runner.model.forward(ctx, runner.views)
+        finally:
+            if collecting:
+                gc.enable()
+
+    def load(self, pieces):
+        self.copied.synchronize()                           # the previous upload has left the staging buffer
+        flat = self.staging.numpy()
+        at = 0
+        for piece, size in zip(pieces, self.sizes):
+            if len(piece) != size:
+                raise RuntimeError('batch layout does not fit the captured graph')
+            flat[at:at + size] = piece
+            at += size
+        self.meta.copy_(self.staging, non_blocking=True)
+        self.copied.record()
+
+    def replay(self, pieces):
+        self.load(pieces)
+        self.graph.replay()
+        return self.logits
+
+
+class DecodeGraphs:
+    def __init__(self, runner):
+        self._runner, self.graphs, self.replays, self.captures = weakref.ref(runner), {}, 0, 0     # no cycle
+
+    @staticmethod
+    def takes(entries):
+        return all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
+                   tuple(e[2] if not isinstance(e, StepEntry) else e.want) == (0,) for e in entries) and len(entries) > 0
+
+    def step(self, entries):
+        runner = self._runner()
+        ps = runner.cache.page_size
+        normal = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2])) for e in entries]
+        runner._validate(normal)
+        longest = max(runner.cache.computed[e.request] for e in normal) + 1
+        bucket = -(-longest // BUCKET) * BUCKET
+        limit = runner.max_positions
+        if limit is not None:
+            bucket = min(bucket, -(-limit // ps) * ps)
+        width = -(-bucket // ps)
+        entries, pieces, facts = runner._describe(normal, table_width=width, validate=False)
+        key = (len(entries), bucket)
+        graph = self.graphs.get(key)
+        if graph is None:
+            if len(self.graphs) >= MAX_GRAPHS:
+                self.graphs.pop(next(iter(self.graphs)))
+            graph = self.graphs[key] = _Graph(runner, entries, pieces, facts, bucket)
+            self.captures += 1
+        logits = graph.replay(pieces).clone()               # the graph's own output buffer is overwritten by the next replay
+        self.replays += 1
+        return logits, entries, facts['starts']

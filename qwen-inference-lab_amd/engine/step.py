@@ -13,12 +13,13 @@ import torch
 
 from ..cache import CacheManager
 from .batch import StepContext, StepEntry
+from .graphs import DecodeGraphs
 
 
 class ModelRunner:
     """Owns the cache of a loaded model and steps batches through it."""
 
-    def __init__(self, model, *, num_pages, page_size=16, max_requests=64, max_step_tokens=None):
+    def __init__(self, model, *, num_pages, page_size=16, max_requests=64, max_step_tokens=None, graphs=True):
         if not model.loaded:
             raise ValueError('the model has no weights yet')
         self.model = model
@@ -28,6 +29,7 @@ class ModelRunner:
                                   max_step_tokens=max_step_tokens)
         self.views = self.cache.views()
         self.steps = 0
+        self.graphs = DecodeGraphs(self) if graphs and self.model.device.type == 'cuda' else None
 
     # -- request lifetime (thin: the cache manager decides)
     def admit(self, request, max_cached_tokens=None):
@@ -61,11 +63,16 @@ class ModelRunner:
             if any(type(w) is not int or not 0 <= w < len(entry.tokens) for w in entry.want):
                 raise ValueError(f'request {entry.request!r}: wanted places must index its tokens')
 
-    def prepare(self, entries):
-        """Pages, then the batch description on the device.  Does not touch the cache contents."""
+    def _describe(self, entries, table_width=None, validate=True):
+        """Pages, then the batch description as host arrays: (entries, pieces, facts).
+
+        pieces: int arrays in a fixed order (tokens, positions, row_seq, cu_seqlens, starts, state
+        slots, logit rows, single rows, then per page group its block tables and token slots).
+        """
         entries = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2]) if len(e) > 2 else ())
                    for e in entries]
-        self._validate(entries)
+        if validate:
+            self._validate(entries)
         cache, ps = self.cache, self.cache.page_size
         starts = [cache.computed[e.request] for e in entries]
         for entry, start in zip(entries, starts):
@@ -80,14 +87,12 @@ class ModelRunner:
         positions = np.arange(n) - cu[row_seq] + np.asarray(starts)[row_seq]
         logit_rows = np.fromiter((cu[i] + w for i, e in enumerate(entries) for w in e.want), dtype=np.int64)
         slots = [cache.slots[e.request] for e in entries]
-        max_context = int(max(st + c for st, c in zip(starts, counts)))
-
         single = cu[:-1][np.asarray(counts) == 1] if max(counts) > 1 else np.zeros(0, dtype=np.int64)
         pieces = [tokens, positions, row_seq, cu, np.asarray(starts), np.asarray(slots), logit_rows, single]
-        group_tables = []
+        widths = []
         for index, group in enumerate(cache.kv_groups):
             tables = [cache.table(index, e.request) for e in entries]
-            width = max(len(t) for t in tables)
+            width = max(len(t) for t in tables) if table_width is None else table_width
             table = np.zeros((s, width), dtype=np.int64)
             for i, t in enumerate(tables):
                 table[i, :len(t)] = t
@@ -95,32 +100,50 @@ class ModelRunner:
             if (table[row_seq, positions // ps] < 0).any():
                 raise RuntimeError('a new token falls into a page that was given back')
             table[table < 0] = 0          # given-back blocks lie outside every window; never read
-            group_tables.append((width, len(pieces)))
+            widths.append(width)
             pieces += [table.reshape(-1), token_slots]
-        flat = np.concatenate(pieces).astype(np.int32)
-        device = torch.from_numpy(flat).to(self.model.device)
-        offsets = np.cumsum([0] + [len(p) for p in pieces])
-        part = lambda i: device[offsets[i]:offsets[i + 1]]
+        facts = dict(n=n, s=s, starts=starts, counts=counts, slots=slots, cu=cu.tolist(), widths=widths,
+                     max_context=int(max(st + c for st, c in zip(starts, counts))), n_logit_rows=len(logit_rows))
+        return entries, pieces, facts
 
+    def _context(self, entries, pieces, facts, device_flat, max_context=None):
+        """StepContext and cache views over a device int32 array holding the pieces back to back."""
+        offsets = np.cumsum([0] + [len(p) for p in pieces])
+        part = lambda i: device_flat[offsets[i]:offsets[i + 1]]
+        s, counts = facts['s'], facts['counts']
         ctx = StepContext(
-            n_tokens=n, n_seqs=s, n_logit_rows=len(logit_rows), token_ids=part(0), positions=part(1),
+            n_tokens=facts['n'], n_seqs=s, n_logit_rows=facts['n_logit_rows'], token_ids=part(0), positions=part(1),
             row_seq=part(2), cu_seqlens=part(3), seq_starts=part(4), seq_slots=part(5), logit_rows=part(6),
-            single_rows=part(7) if max(counts) > 1 else None,
-            max_query=max(counts), max_context=max_context, host_cu_seqlens=cu.tolist(), host_starts=starts,
-            host_slots=slots, requests=[e.request for e in entries])
+            single_rows=part(7) if max(counts) > 1 else None, max_query=max(counts),
+            max_context=max_context or facts['max_context'], host_cu_seqlens=facts['cu'], host_starts=facts['starts'],
+            host_slots=facts['slots'], requests=[e.request for e in entries])
         for view in self.views:
             if view is not None and hasattr(view, 'block_tables'):
-                width, at = group_tables[view.group]
-                view.block_tables = part(at).view(s, width)
+                at = 8 + 2 * view.group
+                view.block_tables = part(at).view(s, facts['widths'][view.group])
                 view.slots = part(at + 1)
-        return entries, ctx
+        return ctx
+
+    def prepare(self, entries):
+        """Pages, then the batch description on the device.  Does not touch the cache contents."""
+        entries, pieces, facts = self._describe(entries)
+        flat = np.concatenate(pieces).astype(np.int32)
+        return entries, self._context(entries, pieces, facts, torch.from_numpy(flat).to(self.model.device))
 
     @torch.inference_mode()
     def step(self, entries):
-        """Run one batch; float32 logits [wanted, vocab] (None if nothing is wanted)."""
-        entries, ctx = self.prepare(entries)
-        logits = self.model.forward(ctx, self.views)
-        for entry, start in zip(entries, ctx.host_starts):
+        """Run one batch; float32 logits [wanted, vocab] (None if nothing is wanted).
+
+        A batch of single decoded tokens that all want their logits replays a captured HIP graph
+        (``graphs.py``) when graphs are enabled; every other batch launches its kernels one by one.
+        """
+        if self.graphs is not None and self.graphs.takes(entries):
+            logits, entries, starts = self.graphs.step(entries)
+        else:
+            entries, ctx = self.prepare(entries)
+            logits = self.model.forward(ctx, self.views)
+            starts = ctx.host_starts
+        for entry, start in zip(entries, starts):
             self.cache.advance(entry.request, start + len(entry.tokens))
         self.steps += 1
         return logits

@@ -203,3 +203,37 @@ def test_long_decoding_crosses_attention_splits(case):
     for t in tokens[200:]:
         got.append(runner.step([StepEntry('r', (t,), (0,))]))
     case.close(torch.cat(got), plain.logits(tokens, weights, config)[199:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_graph_replays_equal_eager_launches(model_folder, dtype):
+    """Decode steps replayed from a captured HIP graph give bit for bit what eager launches give,
+    on every replay, with eager work (a prompt portion of another request) between replays."""
+    config, seed, page_size = CONFIGS['B']
+    folder, weights = model_folder(config, seed)
+    model = load_model(folder, dtype=dtype, device='cuda')
+    runners = [ModelRunner(model, num_pages=24, page_size=page_size, graphs=flag) for flag in (True, False)]
+    prompts = {r: tokens_for(config, n, 60 + n) for r, n in (('a', 21), ('b', 9), ('c', 40))}
+    outputs = [[], []]
+    for which, runner in enumerate(runners):
+        poison(runner)
+        for r in 'ab':
+            runner.admit(r)
+            runner.step([StepEntry(r, tuple(prompts[r][:5]), ())])
+        runner.admit('c')
+        fed = {'a': 5, 'b': 5, 'c': 0}
+        for turn in range(8):
+            batch = [StepEntry(r, (prompts[r][fed[r]],), (0,)) for r in ('b', 'a') if fed[r] < len(prompts[r])]
+            outputs[which].append(runner.step(batch))
+            for entry in batch:
+                fed[entry.request] += 1
+            runner.step([StepEntry('c', tuple(prompts['c'][fed['c']:fed['c'] + 3]), ())])     # eager work in between
+            fed['c'] += 3
+            torch.cuda.synchronize()
+    assert runners[0].graphs.replays >= 8 and runners[0].graphs.captures <= 3
+    for with_graph, eager in zip(*outputs):
+        torch.testing.assert_close(with_graph, eager, atol=0, rtol=0)
+    expected = plain.logits(prompts['a'], weights, config)
+    got = torch.cat([step[1:2] if step.shape[0] == 2 else step[0:1] for step in outputs[0]])[:8].cpu()
+    torch.testing.assert_close(got, expected[5:13], **TOLERANCE[dtype])
