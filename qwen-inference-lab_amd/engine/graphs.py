@@ -71,10 +71,13 @@ class _Graph:
 class DecodeGraphs:
     def __init__(self, runner):
         self._runner, self.graphs, self.replays, self.captures = weakref.ref(runner), {}, 0, 0     # no cycle
+        self._safe = None
 
-    @staticmethod
-    def takes(entries):
-        return all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
+    def takes(self, entries):
+        if self._safe is None:
+            blocks = self._runner().model.blocks
+            self._safe = all(b.mixer is None or b.mixer.graph_safe for b in blocks)
+        return self._safe and all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
                    tuple(e[2] if not isinstance(e, StepEntry) else e.want) == (0,) for e in entries) and len(entries) > 0
 
     def step(self, entries):

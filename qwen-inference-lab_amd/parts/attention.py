@@ -16,6 +16,7 @@ class Attention(Mixer):
     [(heads + 2 kv_heads) head_dim, width] matrix: a pure re-layout, each output
     column is computed from the same row as before.
     """
+    graph_safe = True
 
     def __init__(self, *, width, heads, kv_heads, head_dim, bias, qk_norm_eps, scale,
                  position=None, window=None, dtype=torch.bfloat16):

@@ -103,6 +103,10 @@ class Mixer(Part):
     cache view of its schedule entry (cache/manager.py: KVView or StateView).
     Its result must not depend on how a request's tokens were cut into steps.
     """
+    # True if forward reads only device tensors of the step context (and shapes), never its host
+    # lists: then a decode step may be captured into a HIP graph and replayed with other contents.
+    graph_safe = False
+
     def cache_need(self):
         return None
 

@@ -1,0 +1,135 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice, under random orders of
+requests; reservations; windows giving pages back; state slots."""
+import random
+
+import pytest
+import torch
+
+from qil_amd.cache import CacheManager, CacheFull, PagePool
+from qil_amd.parts import KVNeed, StateNeed
+
+
+def manager(needs=None, pages=4, page_size=2, requests=4, **kwargs):
+    needs = needs or [KVNeed(1, 8, None), KVNeed(1, 8, None)]
+    return CacheManager(needs, num_pages=pages, page_size=page_size, max_requests=requests, allocate=False, **kwargs)
+
+
+def test_reservation_credits_and_reuse():
+    """tests/qil/test_cache.py:11-37: credits do not take physical pages; pages interleave; reuse after release."""
+    cache = manager()
+    assert cache.admit('a', 4) and cache.admit('b', 4)
+    assert cache.free_pages == [4]                       # reserved credits do not consume physical pages
+    assert not cache.admit('c', 1)
+    cache.ensure('a', 1), cache.ensure('b', 1), cache.ensure('a', 4)
+    assert cache.table(0, 'a') == [0, 2] and cache.table(0, 'b') == [1]           # non-contiguous pages
+    with pytest.raises(ValueError):
+        cache.ensure('a', 5)                             # beyond its reservation
+    cache.release('a')
+    assert cache.admit('c', 4)
+    cache.ensure('c', 4)
+    assert cache.table(0, 'c') == [3, 0]                 # FIFO: the never-used page first, then a released one
+    cache.release('b'), cache.release('c')
+    cache.check()
+    assert cache.free_pages == [4] and len(cache.free_slots) == 4
+    with pytest.raises(ValueError):
+        cache.release('c')                               # freed twice
+    with pytest.raises(ValueError):
+        cache.admit('d', 0)
+
+
+def test_unreserved_admission_runs_out_loudly():
+    cache = manager(pages=3)
+    assert cache.admit('a') and cache.admit('b')
+    cache.ensure('a', 4)
+    cache.ensure('b', 2)
+    with pytest.raises(CacheFull):
+        cache.ensure('b', 3)
+    assert cache.table(0, 'b') == [2]                    # all or nothing: nothing was taken
+    cache.check()
+
+
+def test_state_slots_and_duplicates():
+    cache = manager(requests=2)
+    assert cache.admit('a', 2) and cache.admit('b', 2)
+    assert {cache.slots['a'], cache.slots['b']} == {0, 1}
+    assert not cache.admit('c', 2)                       # no slot left, although pages would fit
+    with pytest.raises(ValueError):
+        cache.admit('a', 2)
+    cache.release('a')
+    assert cache.admit('c', 2) and cache.slots['c'] == 0 or cache.slots['c'] == 1
+    cache.check()
+
+
+def test_groups_of_layers_with_different_needs():
+    needs = [KVNeed(2, 16, None), KVNeed(2, 16, 5), KVNeed(2, 16, None), StateNeed((3, 4)), None, ('shared', 1)]
+    cache = CacheManager(needs, num_pages=[6, 5], page_size=2, max_requests=3, dtype=torch.float32, device='cpu',
+                         max_step_tokens=4)
+    assert [g['entries'] for g in cache.kv_groups] == [[0, 2], [1]] and cache.state_groups[0]['entries'] == [3]
+    assert cache.kv_groups[0]['k'].shape == (2, 6, 2, 2, 16) and cache.kv_groups[0]['v'].shape == (2, 6, 2, 16, 2)
+    assert cache.state_groups[0]['state'].shape == (1, 3, 3, 4)
+    views = cache.views()
+    assert views[4] is None and views[5].group == 1 and not views[5].writes and views[3].state.shape == (3, 3, 4)
+    assert cache.admit('r', 12)
+    # the windowed group reserves what a step can hold (window - 1 + step tokens), not the whole length
+    assert cache.kv_groups[1]['pool'].credits['r'] == min(6, (5 - 1 + 4 + 1) // 2 + 1)
+    at = 0
+    for step in (4, 4, 4):
+        cache.ensure('r', at + step)
+        at += step
+        cache.advance('r', at)
+        cache.check()
+    full, window = cache.table(0, 'r'), cache.table(1, 'r')
+    assert len(full) == 6 and all(p >= 0 for p in full)
+    assert window[:4] == [-1, -1, -1, -1] and all(p >= 0 for p in window[4:])    # keys below 12 - 5 + 1 = 8 gave their pages back
+    assert cache.free_pages == [0, 3]
+    cache.release('r')
+    cache.check()
+    assert cache.free_pages == [6, 5]
+
+
+def test_window_never_frees_a_visible_key():
+    pool = PagePool(num_pages=64, page_size=4, window=6)
+    pool.admit('r', None)
+    for computed in range(1, 60):
+        pool.ensure('r', computed)
+        pool.pass_window('r', computed)
+        first_visible = max(0, computed - 6 + 1)          # the next query (position = computed) sees keys > computed - 6
+        assert all(pool.tables['r'][j // 4] >= 0 for j in range(first_visible, computed))
+        assert len(pool.held('r')) <= (6 + 4 - 1) // 4 + 1
+        pool.check()
+
+
+@pytest.mark.parametrize('seed', range(6))
+def test_random_orders_keep_every_page_accounted(seed):
+    r = random.Random(seed)
+    window = r.choice([None, 3, 9])
+    needs = [KVNeed(1, 8, None), KVNeed(1, 8, window)]
+    pages, page_size = r.choice([5, 9, 16]), r.choice([1, 2, 4])
+    cache = CacheManager(needs, num_pages=pages, page_size=page_size, max_requests=4, allocate=False,
+                         max_step_tokens=6)
+    live, finished, name = {}, 0, 0
+    for _ in range(600):
+        action = r.random()
+        if action < 0.25:
+            limit = r.randint(1, pages * page_size)
+            if cache.admit(name, limit):
+                live[name] = limit
+            name += 1
+        elif action < 0.85 and live:
+            request = r.choice(list(live))
+            at = cache.computed[request]
+            if at < live[request]:
+                step = min(r.randint(1, 6), live[request] - at)
+                cache.ensure(request, at + step)          # reserved: must never fail
+                cache.advance(request, at + step)
+        elif live:
+            request = r.choice(list(live))
+            cache.release(request)
+            del live[request]
+            finished += 1
+        cache.check()
+        assert sum(cache.kv_groups[g]['pool'].unreserved for g in range(len(cache.kv_groups))) >= 0
+    for request in list(live):
+        cache.release(request)
+    cache.check()
+    assert cache.free_pages == [pages] * len(cache.kv_groups) and finished > 20

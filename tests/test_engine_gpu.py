@@ -1,0 +1,344 @@
+"""Generation through the entry points, trace replay through bin/trace_run, and a toy architecture,
+on the GPU, against the plain implementation."""
+import json
+import random
+import subprocess
+import sys
+from dataclasses import dataclass
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from conftest import ROOT
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {'A': (plain.TINY_A, 0, 4), 'B': (plain.TINY_B, 1, 8), 'C': (plain.TINY_C, 2, 16)}
+LOGIT_TOLERANCE = {'float32': dict(atol=5e-6, rtol=5e-5), 'bfloat16': dict(atol=0.015, rtol=0.015)}
+# how far below the best float32 logit a chosen token may lie: float32 is exact up to summation
+# order; bfloat16 logits carry errors of a few 1e-3 and may take the other side of a near tie
+# (docs/OPTIMIZATION_DEBUG_LOG.md:101-115 of the reference records such a flip)
+CHOICE_MARGIN = {torch.float32: 1e-5, torch.bfloat16: 0.03}
+
+
+def prompts_for(config, lengths, seed):
+    r = random.Random(seed)
+    return [[r.randrange(config['vocab_size']) for _ in range(n)] for n in lengths]
+
+
+def check_choices(prompt, output, weights, config, dtype, temperature=0.0, seed=0):
+    """Every produced token is the plain sampler's choice on the plain float32 logits of the sequence
+    so far (teacher-forced with the engine's own output), up to the dtype's margin."""
+    logits = plain.logits(prompt + output, weights, config)
+    for index, token in enumerate(output):
+        row = logits[len(prompt) + index - 1]
+        _, scores = plain.sample(row, temperature, seed, index)
+        margin = CHOICE_MARGIN[dtype] / (temperature if temperature else 1.0)
+        assert scores[token] >= scores.max() - margin, (index, token, int(scores.argmax()))
+
+
+@pytest.mark.parametrize('name', sorted(CONFIGS))
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_greedy_generation_through_the_entry_point(model_folder, name, dtype):
+    from qil_amd import Engine, Qwen3
+    config, seed, page_size = CONFIGS[name]
+    folder, weights = model_folder(config, seed)
+    model = Qwen3.from_directory(folder, device='cuda', dtype=dtype)
+    prompts = prompts_for(config, [5, 11, 17, 1], 3)
+    for budget, chunk, pages in ((1, 1, 16), (5, 3, 16), (48, 16, 8)):             # tests/qil/test_engine.py:17
+        engine = Engine(model, num_pages=pages, page_size=page_size, token_budget=budget, prefill_chunk=chunk,
+                        max_active=3)
+        results = engine.generate(prompts, max_new_tokens=8, ignore_eos=True)
+        assert all(r['state'] == 'completed' and r['finish_reason'] == 'length' and len(r['token_ids']) == 8
+                   for r in results)
+        engine.cache.check()
+        assert engine.cache.free_pages == [pages] and engine.idle
+        for prompt, result in zip(prompts, results):
+            if dtype == torch.float32:
+                assert result['token_ids'] == plain.greedy(prompt, 8, weights, config)
+            check_choices(prompt, result['token_ids'], weights, config, dtype)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_temperature_sampling_is_seeded_and_independent_of_the_split(model_folder, dtype):
+    from qil_amd import Engine, Qwen3
+    config, seed, page_size = CONFIGS['B']
+    folder, weights = model_folder(config, seed)
+    model = Qwen3.from_directory(folder, device='cuda', dtype=dtype)
+    prompts = prompts_for(config, [1, 9, 33, 70], 8)
+    outputs = []
+    for budget, chunk in ((48, 16), (7, 3)):
+        engine = Engine(model, num_pages=40, page_size=page_size, token_budget=budget, prefill_chunk=chunk)
+        results = engine.generate(prompts, max_new_tokens=12, ignore_eos=True, temperature=0.8, seed=100)
+        outputs.append([r['token_ids'] for r in results])
+        for index, (prompt, result) in enumerate(zip(prompts, results)):
+            check_choices(prompt, result['token_ids'], weights, config, dtype, temperature=0.8, seed=100 + index)
+    if dtype == torch.float32:
+        assert outputs[0] == outputs[1]                       # the draw does not depend on the work split
+    greedy = Engine(model, num_pages=40, page_size=page_size).generate(prompts, max_new_tokens=12, ignore_eos=True)
+    assert [r['token_ids'] for r in greedy] != outputs[0]
+
+
+def test_eos_stops_and_failure_frees(model_folder, monkeypatch):
+    from qil_amd import Engine, Qwen3
+    config, seed, page_size = CONFIGS['A']
+    folder, weights = model_folder(config, seed)
+    first = plain.greedy([8], 1, weights, config)[0]
+    folder2, _ = model_folder(dict(config, eos_token_id=[first, 255]), seed)
+    model = Qwen3.from_directory(folder2, device='cuda', dtype=torch.float32)
+    engine = Engine(model, num_pages=8, page_size=page_size)
+    result = engine.generate([[8]], max_new_tokens=5)[0]
+    assert result['finish_reason'] == 'eos' and result['token_ids'] == [first]
+    assert len(engine.generate([[8]], max_new_tokens=5, ignore_eos=True)[0]['token_ids']) == 5
+    # non-finite logits fail the batch, free its pages, and later requests still run (qil/engine.py:96-99)
+    from qil_amd import ops
+    real = ops.linear
+    rid = engine.submit([1, 2, 3], max_new_tokens=3, ignore_eos=True)
+    monkeypatch.setattr(ops, 'linear', lambda *a, **k: real(*a, **k) * float('nan') if k.get('out_dtype') == torch.float32 else real(*a, **k))
+    with pytest.raises(RuntimeError, match='non-finite'):
+        engine.step()
+    monkeypatch.setattr(ops, 'linear', real)
+    assert engine.result(rid)['state'] == 'failed' and engine.cache.free_pages == [8]
+    assert engine.generate([[4, 5]], max_new_tokens=2, ignore_eos=True)[0]['state'] == 'completed'
+
+
+def test_command_line(model_folder, tmp_path):
+    config, seed, _ = CONFIGS['A']
+    folder, weights = model_folder(config, seed)
+    prompt = [5, 17, 3, 200, 41]
+    out = tmp_path / 'result.json'
+    run = subprocess.run([sys.executable, '-m', 'qil_amd', '--model', str(folder), '--token-ids', json.dumps(prompt),
+                          '--dtype', 'float32', '--max-new-tokens', '6', '--pages', '8', '--page-size', '4',
+                          '--chunk-size', '2', '--ignore-eos', '--output', str(out)],
+                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    result = json.loads(out.read_text())
+    assert result['token_ids'] == plain.greedy(prompt, 6, weights, config) and result['state'] == 'completed'
+    assert json.loads(run.stdout[run.stdout.index('{'):])['token_ids'] == result['token_ids']
+    random_folder = tmp_path / 'random'
+    run = subprocess.run([sys.executable, '-m', 'qil_amd', '--model', str(random_folder), '--random-config',
+                          json.dumps(plain.TINY_B), '--random-seed', '3', '--token-ids', '[1, 2, 3]', '--dtype', 'bfloat16',
+                          '--max-new-tokens', '4', '--temperature', '0.7', '--seed', '5', '--ignore-eos'],
+                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert len(json.loads(run.stdout[run.stdout.index('{'):])['token_ids']) == 4
+    assert (random_folder / 'model.safetensors').exists()
+
+
+# ------------------------------------------------------------------------------- trace replay
+
+def replay(folder, dtype, steps, out, max_tokens):
+    lines = ''.join(json.dumps(step) + '\n' for step in steps)
+    run = subprocess.run([str(ROOT / 'bin' / 'trace_run'), '--model', str(folder), '--dtype', dtype, '--out', str(out),
+                          '--max-tokens', str(max_tokens)], input=lines, capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-3000:]
+    assert [line for line in run.stdout.splitlines() if line.startswith('done')] == [f"done {s['step']}" for s in steps]
+    return run
+
+
+def collect(out, steps, vocab):
+    """request -> list of (position, logits row) from the files the replay wrote."""
+    fed, rows = {}, {}
+    for step in steps:
+        wanted = sum(len(e['want']) for e in step['entries'])
+        path = Path(out) / f"{step['step']}.f32"
+        assert path.exists() == (wanted > 0)
+        data = np.fromfile(path, dtype='<f4').reshape(wanted, vocab) if wanted else None
+        at = 0
+        for entry in step['entries']:
+            start = fed.get(entry['id'], 0)
+            for w in entry['want']:
+                rows.setdefault(entry['id'], []).append((start + w, torch.from_numpy(data[at].copy())))
+                at += 1
+            fed[entry['id']] = start + len(entry['tokens'])
+        for request in step.get('end', []):
+            fed.pop(request, None)
+    return rows
+
+
+def traces(config, seed):
+    """The four ways of feeding the same requests."""
+    lengths = [70, 45, 83, 38, 64, 51]
+    prompts = {f'r{i}': p for i, p in enumerate(prompts_for(config, lengths, seed))}
+    whole, tail, portions, mixed = [], [], [], []
+    step = 0
+    for name, tokens in prompts.items():                                     # 1: alone and whole
+        whole.append(dict(step=step, entries=[dict(id=name, tokens=tokens, want=list(range(len(tokens))))], end=[name]))
+        step += 1
+    step = 0
+    for name, tokens in list(prompts.items())[:3]:                           # 2: most at once, the last 32 one by one
+        head = len(tokens) - 32
+        tail.append(dict(step=step, entries=[dict(id=name, tokens=tokens[:head], want=list(range(head)))], end=[]))
+        step += 1
+        for i, token in enumerate(tokens[head:]):
+            tail.append(dict(step=step, entries=[dict(id=name, tokens=[token], want=[0])],
+                             end=[name] if i == 31 else []))
+            step += 1
+    r = random.Random(seed)
+    step = 0
+    for name, tokens in list(prompts.items())[:3]:                           # 3: portions of changing size, down to two
+        at = 0
+        while at < len(tokens):
+            size = min(r.choice([2, 2, 3, 7, 16, 5]), len(tokens) - at)
+            portions.append(dict(step=step, entries=[dict(id=name, tokens=tokens[at:at + size], want=list(range(size)))],
+                                 end=[name] if at + size == len(tokens) else []))
+            at += size
+            step += 1
+    waiting, live, step = list(prompts), {}, 0                               # 4: mixed, up to four live, pages reused
+    budget = 256
+    while waiting or live:
+        while waiting and len(live) < 4 and \
+                sum(-(-len(prompts[n]) // 64) * 64 for n in live) + -(-len(prompts[waiting[0]]) // 64) * 64 <= budget:
+            live[waiting.pop(0)] = 0
+        names = list(live)
+        r.shuffle(names)
+        if len(names) > 1 and r.random() < 0.3:
+            names = names[:-1]                                               # a request may sit a step out
+        entries, ended = [], []
+        for name in names:
+            tokens, at = prompts[name], live[name]
+            size = 1 if at >= len(tokens) - 6 else min(r.choice([2, 3, 9, 20]), len(tokens) - 6 - at)
+            want = list(range(size)) if r.random() < 0.8 else []
+            entries.append(dict(id=name, tokens=tokens[at:at + size], want=want))
+            live[name] += size
+            if live[name] == len(tokens):
+                ended.append(name)
+                del live[name]
+        mixed.append(dict(step=step, entries=entries, end=ended))
+        step += 1
+    return prompts, dict(whole=(whole, 128), tail=(tail, 128), portions=(portions, 128), mixed=(mixed, budget))
+
+
+@pytest.mark.parametrize('name', ['B', 'C'])
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_trace_replay_program(model_folder, tmp_path, name, dtype):
+    config, seed, _ = CONFIGS[name]
+    folder, weights = model_folder(config, seed)
+    prompts, shapes = traces(config, seed)
+    expected = {request: plain.logits(tokens, weights, config) for request, tokens in prompts.items()}
+    for shape, (steps, max_tokens) in shapes.items():
+        out = tmp_path / f'{shape}'
+        replay(folder, dtype, steps, out, max_tokens)
+        rows = collect(out, steps, config['vocab_size'])
+        assert rows, shape
+        worst = 0.0
+        for request, items in rows.items():
+            got = torch.stack([row for _, row in items])
+            want = expected[request][[position for position, _ in items]]
+            assert torch.isfinite(got).all()
+            worst = max(worst, (got - want).abs().max().item())
+            torch.testing.assert_close(got, want, **LOGIT_TOLERANCE[dtype], msg=lambda m: f'{shape} {request}: {m}')
+        print(f'{name} {dtype} {shape}: {len(steps)} steps, max abs error {worst:.2e}')
+
+
+# ------------------------------------------------------------------------------- a toy architecture
+
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A mixer with fixed-size per-request state, defined here, becomes an architecture without any
+    change to the framework: a running sum of its inputs, projected.  Chunked steps equal whole ones."""
+    from qil_amd import ops
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.parts import (Mixer, ParamSpec, StateNeed, RMSNorm, GatedMLP, PreNormBlock, Embedding, LMHead,
+                               CausalLM, ScheduleEntry)
+    from qil_amd.registry import register_architecture, read_model_config
+    from qil_amd.weights import write_random_model, load_model
+
+    class RunningSum(Mixer):
+        def __init__(self, width, dtype):
+            super().__init__()
+            self.width, self.dtype = width, dtype
+
+        def param_specs(self):
+            return {'mix.weight': ParamSpec((self.width, self.width))}
+
+        def cache_need(self):
+            return StateNeed((self.width,), 'float32')
+
+        def forward(self, h, ctx, cache):
+            out = torch.empty_like(h, dtype=torch.float32)
+            for s in range(ctx.n_seqs):
+                a, b, slot = ctx.host_cu_seqlens[s], ctx.host_cu_seqlens[s + 1], ctx.host_slots[s]
+                if ctx.host_starts[s] == 0:
+                    cache.state[slot].zero_()                        # a request that starts has no past
+                sums = cache.state[slot] + torch.cumsum(h[a:b].float(), dim=0)
+                counts = torch.arange(ctx.host_starts[s] + 1, ctx.host_starts[s] + b - a + 1, device=h.device)
+                out[a:b] = sums / counts[:, None]
+                cache.state[slot] = sums[-1]
+            return ops.linear(out.to(self.dtype), self.p['mix.weight'], None)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        intermediate_size: int
+        num_hidden_layers: int
+        rms_norm_eps: float = 1e-6
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+        def to_dict(self):
+            return dict(self.__dict__, architectures=['ToyRunningSumLM'], model_type='toy_running_sum')
+
+    def build(config, *, dtype, device):
+        embedding = Embedding(config.vocab_size, config.hidden_size)
+        blocks = [PreNormBlock(mixer_norm=RMSNorm(config.hidden_size, config.rms_norm_eps),
+                               mixer=RunningSum(config.hidden_size, dtype),
+                               ffn_norm=RMSNorm(config.hidden_size, config.rms_norm_eps),
+                               ffn=GatedMLP(width=config.hidden_size, intermediate=config.intermediate_size, dtype=dtype),
+                               dtype=dtype) for _ in range(config.num_hidden_layers)]
+        final_norm, head = RMSNorm(config.hidden_size, config.rms_norm_eps), LMHead(config.vocab_size, config.hidden_size)
+        names = {'embed.weight': (embedding, 'weight'), 'norm.weight': (final_norm, 'weight'), 'head.weight': (head, 'weight')}
+        for i, block in enumerate(blocks):
+            for prefix, part in block.parts().items():
+                for local in part.param_specs():
+                    names[f'layers.{i}.{prefix}.{local}'] = (part, local)
+        return CausalLM(config=config, embedding=embedding, blocks=blocks,
+                        schedule=[ScheduleEntry(i) for i in range(len(blocks))], final_norm=final_norm, head=head,
+                        names=names, dtype=dtype, device=device)
+
+    register_architecture('ToyRunningSumLM', model_type='toy_running_sum', config_class=ToyConfig, build=build,
+                          replace=True)
+    data = dict(architectures=['ToyRunningSumLM'], model_type='toy_running_sum', vocab_size=120, hidden_size=48,
+                intermediate_size=80, num_hidden_layers=2)
+    folder = write_random_model(tmp_path / 'toy', data, seed=4)
+    entry, _ = read_model_config(folder)
+    assert entry.name == 'ToyRunningSumLM'
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+    prompts = prompts_for(data, [19, 8], 6)
+
+    def run(cuts):
+        runner = ModelRunner(model, num_pages=1, page_size=16, max_requests=2)
+        assert runner.graphs is None or not runner.graphs.takes([StepEntry('x', (1,), (0,))])   # host-driven mixer: no graph
+        assert runner.cache.state_groups[0]['state'].shape == (2, 2, 48) and not runner.cache.kv_groups
+        for name in 'ab':
+            runner.admit(name)
+        got, at = {'a': [], 'b': []}, {'a': 0, 'b': 0}
+        for sizes in cuts:
+            entries = []
+            for name, size, tokens in zip('ab', sizes, prompts):
+                if size:
+                    entries.append(StepEntry(name, tuple(tokens[at[name]:at[name] + size]), tuple(range(size))))
+            logits = runner.step(entries)
+            row = 0
+            for entry in entries:
+                got[entry.request].append(logits[row:row + len(entry.tokens)])
+                row += len(entry.tokens)
+                at[entry.request] += len(entry.tokens)
+        return {name: torch.cat(parts) for name, parts in got.items()}
+
+    whole = run([(19, 8)])
+    pieces = run([(5, 1), (2, 1), (7, 1), (1, 1), (4, 4)])
+    for name in 'ab':
+        assert torch.isfinite(whole[name]).all()
+        torch.testing.assert_close(pieces[name], whole[name], atol=1e-5, rtol=1e-4)
+    # the state matters: without the earlier tokens the last logits differ
+    alone = ModelRunner(model, num_pages=1, page_size=16, max_requests=2)
+    alone.admit('z')
+    last = alone.step([StepEntry('z', tuple(prompts[0][-1:]), (0,))])
+    assert not torch.allclose(last[0], whole['a'][-1], atol=1e-3)

@@ -1,0 +1,151 @@
+"""Pins of the plain implementation by what fixes it beside the reference's text: library routines
+in special cases, invariants, and vectors of the reference's own tests.  Each is chosen so that a
+plausible mistake (a wrong sign or pairing, a norm in the wrong place, a wrong head map) fails it."""
+import math
+
+import pytest
+import torch
+from torch.nn import functional as F
+
+import plain_qwen3 as plain
+
+
+def test_rms_norm_is_the_library_routine_in_float32():
+    x, w = torch.randn(5, 24), 1 + 0.3 * torch.randn(24)
+    torch.testing.assert_close(plain.rms_norm(x, w, 1e-6), F.rms_norm(x, (24,), w, 1e-6))
+    # weight multiplies as it is: a zero weight gives zero (rules out 1 + w)
+    assert plain.rms_norm(x, torch.zeros(24), 1e-6).abs().max() == 0
+    # mean square of the output with unit weight is ms / (ms + eps)
+    ms = x.square().mean(-1)
+    torch.testing.assert_close(plain.rms_norm(x, torch.ones(24), 0.5).square().mean(-1), ms / (ms + 0.5))
+
+
+def test_rms_norm_rounds_before_the_weight_in_bfloat16():
+    x = (2 * torch.randn(1, 64)).bfloat16()
+    w = torch.full((64,), 1.00390625 + 2 ** -10)
+    n = x.float() * torch.rsqrt(x.float().square().mean(-1, keepdim=True) + 1e-6)
+    cast_first = n.bfloat16() * w.bfloat16()
+    torch.testing.assert_close(plain.rms_norm(x, w.bfloat16(), 1e-6), cast_first, atol=0, rtol=0)
+
+
+def test_rotation_identity_pairing_sign_and_norm():
+    d = 16
+    x = torch.randn(3, 2, d)
+    zero = plain.rotary_angles(torch.zeros(3, dtype=torch.long), d, 1e4)
+    torch.testing.assert_close(plain.rotate(x, zero), x)                        # position 0: identity
+    unit = torch.zeros(1, 1, d)
+    unit[0, 0, 0] = 1.0
+    out = plain.rotate(unit, plain.rotary_angles(torch.tensor([3]), d, 1.0))      # theta 1: angle = position
+    expected = torch.zeros(d)
+    expected[0], expected[d // 2] = math.cos(3.0), math.sin(3.0)               # pair (0, d/2), + sin below
+    torch.testing.assert_close(out[0, 0], expected)
+    angles = plain.rotary_angles(torch.tensor([7, 90, 511]), d, 1e4)
+    rotated = plain.rotate(x, angles)
+    pair = lambda t: t[..., : d // 2] ** 2 + t[..., d // 2:] ** 2
+    torch.testing.assert_close(pair(rotated), pair(x))                           # each pair keeps its norm
+    # theta -> infinity: only pair 0 rotates
+    big = plain.rotate(x, plain.rotary_angles(torch.tensor([5, 5, 5]), d, 1e300))
+    torch.testing.assert_close(big[..., 1: d // 2], x[..., 1: d // 2])
+    assert not torch.allclose(big[..., 0], x[..., 0])
+
+
+def test_rotated_scores_depend_on_distance_only():
+    d = 32
+    q, k = torch.randn(1, 1, d, dtype=torch.float64), torch.randn(1, 1, d, dtype=torch.float64)
+    def score(m, n):
+        a = plain.rotate(q, plain.rotary_angles(torch.tensor([m]), d, 1e4).double())
+        b = plain.rotate(k, plain.rotary_angles(torch.tensor([n]), d, 1e4).double())
+        return (a * b).sum()
+    torch.testing.assert_close(score(10, 3), score(107, 100), atol=1e-5, rtol=1e-5)
+    assert abs(score(10, 3) - score(3, 10)) > 1e-3                               # sign of the distance matters
+
+
+def test_inverse_frequencies_table_of_the_reference():
+    """qil tests hold that cos/sin rounded to bfloat16 differ between 1 / theta**e and theta**(-e) for
+    head_dim 128, theta 1e6, 2048 positions (tests/qil/test_bf16.py:47-65); the plain table is the former."""
+    inv = plain.inverse_frequencies(128, 1e6)
+    exponent = torch.arange(0, 128, 2, dtype=torch.float32) / 128
+    torch.testing.assert_close(inv, 1.0 / (1e6 ** exponent), atol=0, rtol=0)
+    angles = plain.rotary_angles(torch.arange(2048), 128, 1e6)
+    assert angles.dtype == torch.float32
+    other = torch.arange(2048).float()[:, None] * (1e6 ** (-exponent))[None]
+    assert not torch.equal(other.cos().bfloat16(), angles.cos().bfloat16())
+
+
+@pytest.mark.parametrize('heads,kv_heads', [(4, 4), (6, 2), (5, 1)])
+def test_attention_is_the_library_routine_on_expanded_heads(heads, kv_heads):
+    T, E, d = 5, 12, 8
+    q, k, v = torch.randn(T, heads, d), torch.randn(E, kv_heads, d), torch.randn(E, kv_heads, d)
+    positions = torch.arange(E - T, E)
+    g = heads // kv_heads
+    mask = torch.arange(E)[None, :] <= positions[:, None]
+    expected = F.scaled_dot_product_attention(                                   # qil/model.py:59-68
+        q.transpose(0, 1)[None], k.repeat_interleave(g, 1).transpose(0, 1)[None],
+        v.repeat_interleave(g, 1).transpose(0, 1)[None], attn_mask=mask, scale=d ** -0.5)[0].transpose(0, 1)
+    torch.testing.assert_close(plain.attention(q, k, v, positions, d ** -0.5), expected, atol=1e-6, rtol=1e-5)
+
+
+def test_attention_head_map_causality_and_single_key():
+    heads, kv_heads, d = 6, 2, 4
+    v = torch.zeros(3, kv_heads, d)
+    v[:, 0], v[:, 1] = 1.0, 2.0                                                  # kv heads tell themselves apart
+    out = plain.attention(torch.randn(3, heads, d), torch.randn(3, kv_heads, d), v, torch.arange(3), 0.5)
+    torch.testing.assert_close(out[:, :3], torch.ones(3, 3, d))                  # heads 0-2 read kv head 0 (h // g)
+    torch.testing.assert_close(out[:, 3:], 2 * torch.ones(3, 3, d))
+    q, k, vv = torch.randn(4, heads, d), torch.randn(4, kv_heads, d), torch.randn(4, kv_heads, d)
+    base = plain.attention(q, k, vv, torch.arange(4), 0.5)
+    k2, v2 = k.clone(), vv.clone()
+    k2[3], v2[3] = 9.0, -9.0                                                     # a later token cannot change earlier rows
+    torch.testing.assert_close(plain.attention(q, k2, v2, torch.arange(4), 0.5)[:3], base[:3])
+    first = plain.attention(q[:1], k[:1], vv[:1], torch.tensor([0]), 0.5)
+    torch.testing.assert_close(first[0], vv[0].repeat_interleave(3, 0))           # one visible key: its value
+    windowed = plain.attention(q, k, vv, torch.arange(4), 0.5, window=1)
+    torch.testing.assert_close(windowed, vv.repeat_interleave(3, 1))             # window 1: only the own key
+
+
+def test_mlp_and_block_special_cases():
+    config = dict(plain.TINY_A)
+    weights = plain.random_weights(config, 3)
+    tokens = [5, 17, 3, 200]
+    x = weights['model.embed_tokens.weight'][torch.tensor(tokens)]
+    n = torch.randn(4, 64)
+    g, u, dn = (weights[f'model.layers.0.mlp.{name}_proj.weight'] for name in ('gate', 'up', 'down'))
+    torch.testing.assert_close(plain.gated_mlp(n, g, u, dn), (F.silu(n @ g.T) * (n @ u.T)) @ dn.T)
+    assert plain.gated_mlp(n, torch.zeros_like(g), u, dn).abs().max() == 0       # zero gate: nothing
+    zeroed = dict(weights)
+    for i in range(config['num_hidden_layers']):
+        zeroed[f'model.layers.{i}.self_attn.o_proj.weight'] = torch.zeros_like(weights[f'model.layers.{i}.self_attn.o_proj.weight'])
+        zeroed[f'model.layers.{i}.mlp.down_proj.weight'] = torch.zeros_like(weights[f'model.layers.{i}.mlp.down_proj.weight'])
+    torch.testing.assert_close(plain.hidden_states(tokens, zeroed, config), x)    # pre-norm residual: layers are identity
+
+
+def test_logits_tie_shift_and_last_row():
+    config = dict(plain.TINY_A)
+    weights = plain.random_weights(config, 0)
+    tokens = [1, 7, 4, 8, 12, 5, 2, 9, 3, 11, 6]                                 # tests/qil/test_model.py:22
+    logits = plain.logits(tokens, weights, config)
+    assert logits.shape == (11, 256) and logits.dtype == torch.float32
+    hidden = plain.hidden_states(tokens, weights, config)
+    tied = plain.rms_norm(hidden, weights['model.norm.weight'], 1e-6) @ weights['model.embed_tokens.weight'].T
+    torch.testing.assert_close(logits, tied)                                     # tied head: norm(h) E^T
+    torch.testing.assert_close(plain.logits(tokens[:6], weights, config), logits[:6], atol=1e-6, rtol=1e-5)  # causal
+    untied = dict(config, tie_word_embeddings=False)
+    w2 = dict(weights)
+    w2['lm_head.weight'] = torch.randn(256, 64) * 0.02
+    assert not torch.allclose(plain.logits(tokens, w2, untied), logits)
+    assert plain.greedy([1, 2, 3], 4, weights, config) == plain.greedy([1, 2, 3], 4, weights, config)
+
+
+def test_sampling_reference():
+    row = torch.tensor([0.1, 3.0, 3.0, -1.0])
+    assert plain.sample(row, 0, 0, 0)[0] == 1                                    # tie: lowest index
+    with pytest.raises(RuntimeError):
+        plain.sample(torch.tensor([0.0, float('nan')]), 0, 0, 0)
+    counts = torch.zeros(4)
+    for index in range(3000):
+        counts[plain.sample(row, 0.9, 5, index)[0]] += 1
+    expected = torch.softmax(row / 0.9, 0)
+    assert (counts / 3000 - expected).abs().max() < 0.03
+    assert plain.sample(row, 0.9, 5, 11)[0] == plain.sample(row, 0.9, 5, 11)[0]
+    u = plain.gumbel_uniform(1, 2, 1000)
+    assert 0 < u.min() and u.max() < 1 and abs(u.mean() - 0.5) < 0.05
