@@ -142,7 +142,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        packed[jt * 2 + i] = (uint32_t)f32_to_bf16(s[jt][2 * i]) | ((uint32_t)f32_to_bf16(s[jt][2 * i + 1]) << 16);
+        packed[jt * 2 + i] = pack_bf16(s[jt][2 * i], s[jt][2 * i + 1]);
     const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
     const uint32_t mask[4] = {keep[0][0] | (keep[0][1] << 16), keep[0][2] | (keep[0][3] << 16),
                               keep[1][0] | (keep[1][1] << 16), keep[1][2] | (keep[1][3] << 16)};

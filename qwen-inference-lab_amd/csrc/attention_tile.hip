@@ -11,7 +11,7 @@
 // A row at absolute position p sees key j iff j <= p, and j > p - window with a window
 // (qil/model.py:62-64).  Keys at or beyond the block's last position + 1 are never loaded: they
 // are not written yet or belong to nobody; their LDS slots are zero so that 0 * garbage cannot
-// make a NaN.
+// make a NaN.  A wave skips key sub-tiles that lie wholly in the future of all its rows.
 //
 // Matrix-core formulation (wave64, 16x16 tiles).  Scores are computed transposed,
 //   S^T[key, row] = sum_dim K[key, dim] Q[row, dim]        A = K tile (LDS), B = Q (registers)
@@ -40,15 +40,22 @@ template <> struct TileTraits<float> {
   static constexpr int PAD = 4;
 };
 
-__device__ __forceinline__ float softmax_exp(float x, bf16_t) { return __builtin_amdgcn_exp2f(x * 1.44269504088896f); }
-__device__ __forceinline__ float softmax_exp(float x, float) { return expf(x); }
+// exp(scale * (x - base)): one fused multiply-add and the hardware's exp2 for bfloat16; the library's
+// exp on an exactly rounded argument for float32.
+__device__ __forceinline__ float scaled_exp(float x, float base, float scale, bf16_t) {
+  const float c = scale * 1.44269504088896f;
+  return __builtin_amdgcn_exp2f(fmaf(x, c, -base * c));
+}
+__device__ __forceinline__ float scaled_exp(float x, float base, float scale, float) { return expf((x - base) * scale); }
 
-template <typename T, int DMAX>
-__global__ void __launch_bounds__(TILE_THREADS)
+// RB: 16-row tiles per wave.  A K or V^T fragment read from LDS serves RB products, which is what
+// keeps the kernel from being bound by LDS reads.
+template <typename T, int DMAX, int RB>
+__global__ void __launch_bounds__(TILE_THREADS, 2)
 attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                  const int* __restrict__ block_tables, int table_stride, const int* __restrict__ cu_seqlens,
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
-                 int page_size, int window, float scale, int GH, int chunks) {
+                 int page_size, int window, float scale, int GH, int chunks, int ps_shift) {
   using TT = TileTraits<T>;
   constexpr int BK = TT::BK, KSTEP = TT::KSTEP, PAD = TT::PAD;
   constexpr bool BF16 = sizeof(T) == 2;
@@ -60,19 +67,26 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
   const int seq = blockIdx.y;
   const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
   if (n < 2) return;
-  const int RT = 4 / GH;
-  const int tile_row0 = blockIdx.x * 16 * RT;
+  const int RT = 4 / GH;                        // waves along rows
+  const int block_rows = 16 * RB * RT;
+  // Later rows see more keys.  Blocks are handed to the 256 CUs in launch order, so consecutive groups
+  // of 256 blocks walk the row tiles in opposite directions: a CU that got a long block gets a short one.
+  // (The direction is fixed per (sequence, head group), so every row tile is still served exactly once.)
+  const int linear = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int across = ((linear >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int tile_row0 = across * block_rows;
   if (tile_row0 >= n) return;
   const int kvh = blockIdx.z / chunks, chunk = blockIdx.z % chunks;
   const int g = heads / kv_heads;
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int head_local = chunk * GH + wave % GH, row_tile = wave / GH;
-  const bool wave_active = head_local < g && tile_row0 + row_tile * 16 < n;
+  const int head_local = chunk * GH + wave % GH, row_group = wave / GH;
+  const int wave_row0 = tile_row0 + row_group * 16 * RB;
+  const bool wave_active = head_local < g && wave_row0 < n;
   const int head = kvh * g + head_local;
   const int start = seq_starts[seq];
 
-  const int rows_in_block = min(16 * RT, n - tile_row0);
+  const int rows_in_block = min(block_rows, n - tile_row0);
   const int pos_first = start + tile_row0;
   const int key_end = pos_first + rows_in_block;                       // last position + 1
   const int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
@@ -83,79 +97,182 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
   const int v_row = BK + PAD;                                          // elements per V^T row in LDS
   T* Ks = reinterpret_cast<T*>(lds_raw);                               // [BK][k_row]
   T* Vt = Ks + BK * k_row;                                             // [dt * 16][v_row]
-
-  const int my_row = tile_row0 + row_tile * 16 + r;
-  const bool row_valid = wave_active && my_row < n;
-  const int my_pos = start + my_row;
   const int* table = block_tables + (size_t)seq * table_stride;
 
-  // ---- Q fragments: B operand, Q[row r][dims of this lane's k slots]
-  bf16x8 qb[BF16 ? QFRAGS : 1];
-  float qf[BF16 ? 1 : QFRAGS];
-  {
-    const T* qrow = q + (size_t)(q0 + (row_valid ? my_row : 0)) * q_stride + (size_t)(wave_active ? head : 0) * d;
+  int my_row[RB], my_pos[RB];
+  bool row_valid[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    my_row[b] = wave_row0 + b * 16 + r;
+    row_valid[b] = wave_active && my_row[b] < n;
+    my_pos[b] = start + my_row[b];
+  }
+  const int wave_last_pos = start + min(n, wave_row0 + 16 * RB) - 1;   // nothing beyond it is visible to this wave
+
+  // ---- Q fragments: B operands, Q[row r of tile b][dims of this lane's k slots]
+  bf16x8 qb[RB][BF16 ? QFRAGS : 1];
+  float qf[RB][BF16 ? 1 : QFRAGS];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const T* qrow = q + (size_t)(q0 + (row_valid[b] ? my_row[b] : 0)) * q_stride + (size_t)(wave_active ? head : 0) * d;
     if constexpr (BF16) {
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks) {
         const int dim = ks * 32 + kb * 8;
         uint4 raw = make_uint4(0, 0, 0, 0);
-        if (row_valid && dim < d) raw = *reinterpret_cast<const uint4*>(qrow + dim);
-        qb[ks] = __builtin_bit_cast(bf16x8, raw);
+        if (row_valid[b] && dim < d) raw = *reinterpret_cast<const uint4*>(qrow + dim);
+        qb[b][ks] = __builtin_bit_cast(bf16x8, raw);
       }
     } else {
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks) {
         const int dim = ks * 4 + kb;
-        qf[ks] = (row_valid && dim < d) ? qrow[dim] : 0.f;
+        qf[b][ks] = (row_valid[b] && dim < d) ? qrow[dim] : 0.f;
       }
     }
   }
 
-  float m = -INFINITY, l = 0.f;
-  f32x4 o[DTILES];
+  float m[RB], l[RB];
+  f32x4 o[RB][DTILES];
 #pragma unroll
-  for (int t = 0; t < DTILES; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < RB; ++b) {
+    m[b] = -INFINITY;
+    l[b] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DTILES; ++t) o[b][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
 
+  // ---- what this thread stages of every tile (the same places each time; only the keys move on)
   const int vec_per_key = (dt * 16) / 8;               // 8-element vectors per key covering the dim tiles
-  for (int k0 = key_begin / BK * BK; k0 < key_end; k0 += BK) {
+  const bool fast_v = page_size % 8 == 0;              // 8 keys of a dim are 16 (32) contiguous bytes of a V page
+  constexpr int K_ITERS = (BK * (DMAX / 8) + TILE_THREADS - 1) / TILE_THREADS;
+  constexpr int V_ITERS = (DMAX * (BK / 8) + TILE_THREADS - 1) / TILE_THREADS;
+  int k_kl[K_ITERS], k_dv[K_ITERS], v_grp[V_ITERS], v_dim[V_ITERS];
+#pragma unroll
+  for (int it = 0; it < K_ITERS; ++it) {
+    const int idx = threadIdx.x + it * TILE_THREADS;
+    k_kl[it] = idx < BK * vec_per_key ? idx / vec_per_key : -1;
+    k_dv[it] = (idx - max(k_kl[it], 0) * vec_per_key) * 8;
+  }
+#pragma unroll
+  for (int it = 0; it < V_ITERS; ++it) {
+    const int idx = threadIdx.x + it * TILE_THREADS;
+    v_grp[it] = idx < dt * 16 * (BK / 8) ? idx / (dt * 16) : -1;         // consecutive threads: consecutive dims
+    v_dim[it] = idx - max(v_grp[it], 0) * (dt * 16);
+  }
+  auto page_of = [&](int key, int& offset) -> size_t {
+    int block;
+    if (ps_shift >= 0) { block = key >> ps_shift; offset = key & (page_size - 1); }
+    else { block = key / page_size; offset = key - block * page_size; }
+    return (size_t)table[block];
+  };
+
+  // Fast staging (bfloat16, page_size % 8 == 0): no branch around a load, so that all table lookups of
+  // a tile go out together, then all K and V^T vectors, and the zeroing of invisible keys is a select.
+  // Addresses of places that are not needed are clamped onto needed ones.
+  const bool fast = BF16 && fast_v;
+  const int first_tile = key_begin / BK * BK;
+
+  for (int k0 = first_tile; k0 < key_end; k0 += BK) {
     __syncthreads();                                   // the previous tile is consumed
-    // ---- stage K (row major) and V (transposed) of keys [k0, k0 + BK)
-    for (int idx = threadIdx.x; idx < BK * vec_per_key; idx += TILE_THREADS) {
-      const int kl = idx / vec_per_key, dv = (idx - kl * vec_per_key) * 8;
-      const int key = k0 + kl;
+    if (fast) {
+      if constexpr (BF16) {
+        const bool inside = k0 >= key_begin && k0 + BK <= key_end;          // no key of the tile needs zeroing
+        size_t k_page[K_ITERS], v_page[V_ITERS];
+        int k_off[K_ITERS], v_off[V_ITERS];
+#pragma unroll
+        for (int it = 0; it < K_ITERS; ++it) {
+          const int key = min(max(k0 + max(k_kl[it], 0), key_begin), key_end - 1);
+          k_page[it] = page_of(key, k_off[it]);
+        }
+#pragma unroll
+        for (int it = 0; it < V_ITERS; ++it) {
+          const int key = min(max(k0 + max(v_grp[it], 0) * 8, key_begin & ~7), (key_end - 1) & ~7);
+          v_page[it] = page_of(key, v_off[it]);
+        }
+        uint4 k_reg[K_ITERS], v_reg[V_ITERS];
+#pragma unroll
+        for (int it = 0; it < K_ITERS; ++it)
+          k_reg[it] = *reinterpret_cast<const uint4*>(
+              k_cache + ((k_page[it] * kv_heads + kvh) * page_size + k_off[it]) * (size_t)d + min(k_dv[it], d - 8));
+#pragma unroll
+        for (int it = 0; it < V_ITERS; ++it)
+          v_reg[it] = *reinterpret_cast<const uint4*>(
+              v_cache + ((v_page[it] * kv_heads + kvh) * (size_t)d + min(v_dim[it], d - 1)) * page_size + v_off[it]);
+#pragma unroll
+        for (int it = 0; it < K_ITERS; ++it) {
+          if (k_kl[it] < 0) continue;
+          const int key = k0 + k_kl[it];
+          const bool valid = key >= key_begin && key < key_end && k_dv[it] < d;
+          *reinterpret_cast<uint4*>(Ks + k_kl[it] * k_row + k_dv[it]) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int it = 0; it < V_ITERS; ++it) {
+          if (v_grp[it] < 0) continue;
+          uint4 raw = v_dim[it] < d ? v_reg[it] : make_uint4(0, 0, 0, 0);
+          if (!inside) {   // zero what lies outside [key_begin, key_end): never written, or someone else's
+            const int key = k0 + v_grp[it] * 8;
+            uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (!(key + e >= key_begin && key + e < key_end)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            raw = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+          *reinterpret_cast<uint4*>(Vt + v_dim[it] * v_row + v_grp[it] * 8) = raw;
+        }
+      }
+    } else {
+    // ---- stage K (row major) of keys [k0, k0 + BK); V too on the generic path
+#pragma unroll
+    for (int it = 0; it < K_ITERS; ++it) {
+      if (k_kl[it] < 0) continue;
+      const int kl = k_kl[it], dv = k_dv[it], key = k0 + kl;
       const bool valid = key >= key_begin && key < key_end && dv < d;
       T* kdst = Ks + kl * k_row + dv;
+      size_t page = 0;
+      int offset = 0;
+      if (valid) page = page_of(key, offset);
+      const size_t kbase = ((page * kv_heads + kvh) * page_size + offset) * (size_t)d + dv;
+      const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + dv) * page_size + offset;
       if constexpr (BF16) {
-        uint4 kraw = make_uint4(0, 0, 0, 0), vraw = make_uint4(0, 0, 0, 0);
-        if (valid) {
-          const size_t page = table[key / page_size];
-          const size_t base = ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d + dv;
-          kraw = *reinterpret_cast<const uint4*>(k_cache + base);
-          const bf16_t* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + dv) * page_size + (key % page_size);
-          uint32_t w[4] = {0, 0, 0, 0};
-#pragma unroll
-          for (int e = 0; e < 8; ++e) w[e >> 1] |= (uint32_t)column[(size_t)e * page_size] << ((e & 1) * 16);
-          vraw = make_uint4(w[0], w[1], w[2], w[3]);
-        }
+        uint4 kraw = make_uint4(0, 0, 0, 0);
+        if (valid) kraw = *reinterpret_cast<const uint4*>(k_cache + kbase);
         *reinterpret_cast<uint4*>(kdst) = kraw;
-        const uint32_t w[4] = {vraw.x, vraw.y, vraw.z, vraw.w};
+        if (!fast_v) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(dv + e) * v_row + kl] = (bf16_t)(w[e >> 1] >> ((e & 1) * 16));
+          for (int e = 0; e < 8; ++e) Vt[(dv + e) * v_row + kl] = valid ? column[(size_t)e * page_size] : (bf16_t)0;
+        }
       } else {
-        float kv8[8], vv8[8];
+        float kv8[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { kv8[e] = 0.f; vv8[e] = 0.f; }
-        if (valid) {
-          const size_t page = table[key / page_size];
-          const size_t base = ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d + dv;
-          ld8(k_cache + base, kv8);
-          const float* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + dv) * page_size + (key % page_size);
+        for (int e = 0; e < 8; ++e) kv8[e] = 0.f;
+        if (valid) ld8(k_cache + kbase, kv8);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) vv8[e] = column[(size_t)e * page_size];
+        for (int e = 0; e < 8; ++e) kdst[e] = kv8[e];
+        if (!fast_v) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) Vt[(dv + e) * v_row + kl] = valid ? column[(size_t)e * page_size] : 0.f;
+        }
+      }
+    }
+    if (fast_v) {
+      // ---- stage V^T: a thread copies 8 consecutive keys of one dim (one vector of the page's row)
+#pragma unroll
+      for (int it = 0; it < V_ITERS; ++it) {
+        if (v_grp[it] < 0) continue;
+        const int grp = v_grp[it], dim = v_dim[it], key = k0 + grp * 8;
+        T* dst = Vt + dim * v_row + grp * 8;
+        const bool any = key + 7 >= key_begin && key < key_end && dim < d;
+        float vals[8];
+        if (any) {
+          int offset;
+          const size_t page = page_of(key, offset);
+          ld8(v_cache + ((page * kv_heads + kvh) * (size_t)d + dim) * page_size + offset, vals);
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { kdst[e] = kv8[e]; Vt[(dv + e) * v_row + kl] = vv8[e]; }
+        for (int e = 0; e < 8; ++e) dst[e] = (any && key + e >= key_begin && key + e < key_end) ? vals[e] : 0.f;
       }
+    }
     }
     if constexpr (BF16) {
       // K rows are read in steps of 32 dims: zero the tail between the dim tiles and the padded width
@@ -165,73 +282,101 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
           Ks[(idx / tail) * k_row + tail0 + idx % tail] = 0;
     }
     __syncthreads();
-    if (!wave_active) continue;
+    if (!wave_active || k0 > wave_last_pos) continue;
 
-    // ---- S^T = K Q^T for the tile's 16-key sub-tiles
-    f32x4 s[SUB];
+    // ---- S^T = K Q^T for the tile's 16-key sub-tiles, each K fragment serving the RB row tiles
+    f32x4 s[RB][SUB];
 #pragma unroll
     for (int jt = 0; jt < SUB; ++jt) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int b = 0; b < RB; ++b) s[b][jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (k0 + jt * 16 > wave_last_pos) continue;                     // wholly in the future of every row
       const T* krow = Ks + (jt * 16 + r) * k_row;
       if constexpr (BF16) {
 #pragma unroll
         for (int ks = 0; ks < QFRAGS; ++ks) {
           if (ks * 32 < d) {
             const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + ks * 32 + kb * 8));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ks], acc, 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[b][ks], s[b][jt], 0, 0, 0);
           }
         }
       } else {
 #pragma unroll
         for (int ks = 0; ks < QFRAGS; ++ks)
-          if (ks * 4 < d) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(krow[ks * 4 + kb], qf[ks], acc, 0, 0, 0);
+          if (ks * 4 < d) {
+            const float a = krow[ks * 4 + kb];
+#pragma unroll
+            for (int b = 0; b < RB; ++b) s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, qf[b][ks], s[b][jt], 0, 0, 0);
+          }
       }
-      s[jt] = acc;
     }
-    // ---- mask, scale, online softmax (per-lane row statistics)
-    float mx = -INFINITY;
+    // ---- mask and online softmax (per-lane row statistics).  m holds the running maximum of the RAW
+    // scores; the scale (> 0) enters once, in the exponent: p = exp(scale * (s - m)).
+    // every key of the tile is visible to every row of the wave unless the tile touches the wave's
+    // first row's future, the window's edge or the rows beyond the sequence
+    const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 16 * RB <= n &&
+                             (window <= 0 || k0 > wave_last_pos - window);
 #pragma unroll
-    for (int jt = 0; jt < SUB; ++jt)
+    for (int b = 0; b < RB; ++b) {
+      float mx = -INFINITY;
+      if (all_visible) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + jt * 16 + 4 * kb + i;
-        const bool visible = row_valid && key <= my_pos && (window <= 0 || key > my_pos - window);
-        const float v = visible ? s[jt][i] * scale : -INFINITY;
-        s[jt][i] = v;
-        mx = fmaxf(mx, v);
+        for (int jt = 0; jt < SUB; ++jt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[b][jt][i]);
+      } else {
+#pragma unroll
+        for (int jt = 0; jt < SUB; ++jt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = k0 + jt * 16 + 4 * kb + i;
+            const bool visible = row_valid[b] && key <= my_pos[b] && (window <= 0 || key > my_pos[b] - window);
+            const float v = visible ? s[b][jt][i] : -INFINITY;
+            s[b][jt][i] = v;
+            mx = fmaxf(mx, v);
+          }
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = (m_new == -INFINITY) ? 1.f : softmax_exp(m - m_new, T());   // m = -inf gives 0
-    float psum = 0.f;
+      mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+      const float m_new = fmaxf(m[b], mx);
+      const float base = (m_new == -INFINITY) ? 0.f : m_new;                              // exp(-inf - 0) = 0
+      const float alpha = (m_new == -INFINITY) ? 1.f : scaled_exp(m[b], base, scale, T());  // m = -inf gives 0
+      float psum = 0.f;
 #pragma unroll
-    for (int jt = 0; jt < SUB; ++jt)
+      for (int jt = 0; jt < SUB; ++jt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = (s[jt][i] == -INFINITY) ? 0.f : softmax_exp(s[jt][i] - m_new, T());
-        s[jt][i] = p;
-        psum += p;
+        for (int i = 0; i < 4; ++i) {
+          const float p = scaled_exp(s[b][jt][i], base, scale, T());
+          s[b][jt][i] = p;
+          psum += p;
+        }
+      l[b] = l[b] * alpha + psum;
+      if (m_new != m[b]) {                       // nothing to rescale while the maximum stands
+#pragma unroll
+        for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[b][t][i] *= alpha;
       }
-    l = l * alpha + psum;
-    m = m_new;
-#pragma unroll
-    for (int t = 0; t < DTILES; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+      m[b] = m_new;
+    }
 
-    // ---- O^T += V^T P^T
+    // ---- O^T += V^T P^T, each V^T fragment serving the RB row tiles
     if constexpr (BF16) {
 #pragma unroll
       for (int st = 0; st < SUB / 2; ++st) {
-        uint32_t packed[4];
+        if (k0 + st * 32 > wave_last_pos) continue;
+        bf16x8 pb[RB];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          packed[i] = (uint32_t)f32_to_bf16(s[2 * st][2 * i]) | ((uint32_t)f32_to_bf16(s[2 * st][2 * i + 1]) << 16);
-          packed[2 + i] = (uint32_t)f32_to_bf16(s[2 * st + 1][2 * i]) |
-                          ((uint32_t)f32_to_bf16(s[2 * st + 1][2 * i + 1]) << 16);
+        for (int b = 0; b < RB; ++b) {
+          uint32_t packed[4];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            packed[i] = pack_bf16(s[b][2 * st][2 * i], s[b][2 * st][2 * i + 1]);
+            packed[2 + i] = pack_bf16(s[b][2 * st + 1][2 * i], s[b][2 * st + 1][2 * i + 1]);
+          }
+          pb[b] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
         }
-        const bf16x8 b = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
 #pragma unroll
         for (int t = 0; t < DTILES; ++t) {
           if (t < dt) {
@@ -239,39 +384,48 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
             const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
             const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
             const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, o[t], 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) o[b][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[b], o[b][t], 0, 0, 0);
           }
         }
       }
     } else {
 #pragma unroll
-      for (int jt = 0; jt < SUB; ++jt)
+      for (int jt = 0; jt < SUB; ++jt) {
+        if (k0 + jt * 16 > wave_last_pos) continue;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int t = 0; t < DTILES; ++t)
-            if (t < dt)
-              o[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(Vt[(t * 16 + r) * v_row + jt * 16 + 4 * kb + i], s[jt][i],
-                                                          o[t], 0, 0, 0);
+            if (t < dt) {
+              const float a = Vt[(t * 16 + r) * v_row + jt * 16 + 4 * kb + i];
+#pragma unroll
+              for (int b = 0; b < RB; ++b) o[b][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, s[b][jt][i], o[b][t], 0, 0, 0);
+            }
+      }
     }
   }
 
   if (!wave_active) return;
-  l += __shfl_xor(l, 16, QIL_WAVE);
-  l += __shfl_xor(l, 32, QIL_WAVE);
-  if (!row_valid) return;
-  const float inv = 1.f / l;
-  T* orow = out + ((size_t)(q0 + my_row) * heads + head) * d;
 #pragma unroll
-  for (int t = 0; t < DTILES; ++t)
+  for (int b = 0; b < RB; ++b) {
+    float total = l[b];
+    total += __shfl_xor(total, 16, QIL_WAVE);
+    total += __shfl_xor(total, 32, QIL_WAVE);
+    if (!row_valid[b]) continue;
+    const float inv = 1.f / total;
+    T* orow = out + ((size_t)(q0 + my_row[b]) * heads + head) * d;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int dim = t * 16 + 4 * kb + i;
-      if (dim < d) st(orow + dim, o[t][i] * inv);
-    }
+    for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int dim = t * 16 + 4 * kb + i;
+        if (dim < d) st(orow + dim, o[b][t][i] * inv);
+      }
+  }
 }
 
-template <typename T, int DMAX>
+template <typename T, int DMAX, int RB>
 static int launch_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                        int max_query, int heads, int kv_heads, int d, int page_size, int window, float scale,
@@ -282,17 +436,20 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
   const bool bf16 = sizeof(T) == 2;
   const int k_row = (bf16 ? (d + 31) / 32 * 32 : (d + 15) / 16 * 16) + TT::PAD, v_row = TT::BK + TT::PAD;
   const size_t lds = ((size_t)TT::BK * k_row + (size_t)((d + 15) / 16 * 16) * v_row) * sizeof(T);
-  auto kernel = attn_tile_kernel<T, DMAX>;
+  auto kernel = attn_tile_kernel<T, DMAX, RB>;
   static size_t granted = 0;                     // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     granted = lds;
   }
-  dim3 grid((max_query + 16 * RT - 1) / (16 * RT), n_seqs, kv_heads * chunks);
+  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks);
+  int ps_shift = -1;                                      // log2 of a power-of-two page size
+  for (int b = 0; b < 30; ++b)
+    if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(TILE_THREADS), lds, s, (const T*)q, q_stride, (const T*)k_cache,
                      (const T*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (T*)out, heads, kv_heads, d,
-                     page_size, window, scale, GH, chunks);
+                     page_size, window, scale, GH, chunks, ps_shift);
   return (int)hipGetLastError();
 }
 
@@ -305,7 +462,7 @@ extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, c
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
 #define QIL_TILE_CASE(T, DMAX)                                                                                      \
-  return launch_tile<T, DMAX>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
+  return launch_tile<T, DMAX, (sizeof(T) == 2 && DMAX <= 128) ? 2 : 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s)
   if (dtype == QIL_F32) {
     if (d <= 64) QIL_TILE_CASE(float, 64);

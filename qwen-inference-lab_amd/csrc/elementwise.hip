@@ -20,8 +20,7 @@ __device__ __forceinline__ float4 load4(const bf16_t* p) {
 }
 __device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
-  *reinterpret_cast<uint2*>(p) = make_uint2((uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
-                                            (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16));
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
 }
 
 // A sub-layer's output arrives either in the model's type T (one array) or as float32 partial sums
@@ -142,6 +141,21 @@ __global__ void silu_mul_kernel(const TD* __restrict__ gate_up, int splits, size
   st(out + idx, (g / (1.f + expf(-g))) * u);
 }
 
+// Four outputs a thread, vector loads and stores; inner % 4 == 0.
+template <typename TD, typename T>
+__global__ void silu_mul_vec_kernel(const TD* __restrict__ gate_up, int splits, size_t split_stride,
+                                    T* __restrict__ out, int inner, size_t total4) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total4) return;
+  const int per_row = inner / 4;
+  const size_t n = idx / per_row;
+  const int i = (int)(idx - n * per_row) * 4;
+  const float4 g = load_sum4(gate_up, n * 2 * (size_t)inner + i, splits, split_stride);
+  const float4 u = load_sum4(gate_up, n * 2 * (size_t)inner + inner + i, splits, split_stride);
+  store4(out + n * (size_t)inner + i, make_float4((g.x / (1.f + expf(-g.x))) * u.x, (g.y / (1.f + expf(-g.y))) * u.y,
+                                                  (g.z / (1.f + expf(-g.z))) * u.z, (g.w / (1.f + expf(-g.w))) * u.w));
+}
+
 // x[n, i] += bias[i]
 template <typename T>
 __global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int width, size_t total) {
@@ -205,18 +219,27 @@ int qil_silu_mul(const void* gate_up, int in_dtype, int splits, void* out, int n
   if (total == 0) return 0;
   if (splits < 1 || (in_dtype == QIL_BF16 && splits != 1)) return -1;
   const size_t stride = (size_t)n * 2 * inner;
-  const unsigned blocks = (unsigned)((total + 255) / 256);
+  const bool vec = inner % 4 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0);
+  const size_t work = vec ? total / 4 : total;
+  const unsigned blocks = (unsigned)((work + 255) / 256);
+#define QIL_SILU_CASE(TD, T)                                                                                          \
+  do {                                                                                                                \
+    if (vec)                                                                                                          \
+      hipLaunchKernelGGL((silu_mul_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)gate_up, splits,      \
+                         stride, (T*)out, inner, work);                                                               \
+    else                                                                                                              \
+      hipLaunchKernelGGL((silu_mul_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)gate_up, splits, stride,  \
+                         (T*)out, inner, total);                                                                      \
+  } while (0)
   if (out_dtype == QIL_F32) {
     if (in_dtype != QIL_F32) return -1;
-    hipLaunchKernelGGL((silu_mul_kernel<float, float>), dim3(blocks), dim3(256), 0, s, (const float*)gate_up, splits,
-                       stride, (float*)out, inner, total);
+    QIL_SILU_CASE(float, float);
   } else if (in_dtype == QIL_F32) {
-    hipLaunchKernelGGL((silu_mul_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, s, (const float*)gate_up, splits,
-                       stride, (bf16_t*)out, inner, total);
+    QIL_SILU_CASE(float, bf16_t);
   } else {
-    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, s, (const bf16_t*)gate_up, splits,
-                       stride, (bf16_t*)out, inner, total);
+    QIL_SILU_CASE(bf16_t, bf16_t);
   }
+#undef QIL_SILU_CASE
   QIL_RETURN_LAUNCH_STATUS();
 }
 
