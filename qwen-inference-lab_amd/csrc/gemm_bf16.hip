@@ -63,7 +63,35 @@ gemm_bf16_stream_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
     for (int j = 0; j < NT; ++j) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   const int k_begin = split * steps_per_split * 32, k_end = min(K, k_begin + steps_per_split * 32);
-  for (int kc = k_begin; kc < k_end; kc += chunk) {
+  // W fragments of the next UNROLL k steps are always in flight: the first group is requested before A
+  // is even staged, and each later group before the products of the group in hand.  Two register
+  // buffers take turns; the loop is written out in pairs so that each is indexed statically.
+  uint4 b0[UNROLL][NT], b1[UNROLL][NT];
+  auto request = [&](uint4 (&b)[UNROLL][NT], int k0) {     // k steps starting at column k0
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = k0 + u * 32 + kb * 8;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) b[u][j] = load_frag<ALIGNED>(W, n0 + j * 16 + r, N, k < k_end ? k : K, K);
+    }
+  };
+  auto multiply = [&](const uint4 (&b)[UNROLL][NT], int step, int steps) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (step + u < steps) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const uint4 a = *reinterpret_cast<const uint4*>(a_lds + (t * 16 + r) * row_width + (step + u) * 32 + kb * 8);
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                __builtin_bit_cast(bf16x8, b[u][j]), acc[t][j], 0, 0, 0);
+        }
+      }
+    }
+  };
+  request(b0, k_begin);
+  for (int kc = k_begin; kc < k_end; kc += chunk) {          // chunk is a multiple of 64 * UNROLL columns
     const int width = min(chunk, k_end - kc);               // columns of this chunk (last one may be short)
     __syncthreads();                                        // the previous chunk is consumed
     for (int idx = threadIdx.x; idx < 16 * MT * (chunk / 8); idx += GEMM_WAVES * QIL_WAVE) {
@@ -73,27 +101,11 @@ gemm_bf16_stream_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
     }
     __syncthreads();
     const int steps = (width + 31) / 32;
-    for (int step = 0; step < steps; step += UNROLL) {
-      uint4 b[UNROLL][NT];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const int k = (step + u < steps) ? kc + (step + u) * 32 + kb * 8 : K;    // K: out of range, loads nothing
-#pragma unroll
-        for (int j = 0; j < NT; ++j) b[u][j] = load_frag<ALIGNED>(W, n0 + j * 16 + r, N, k, K);
-      }
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        if (step + u < steps) {
-#pragma unroll
-          for (int t = 0; t < MT; ++t) {
-            const uint4 a = *reinterpret_cast<const uint4*>(a_lds + (t * 16 + r) * row_width + (step + u) * 32 + kb * 8);
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-              acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
-                                                                  __builtin_bit_cast(bf16x8, b[u][j]), acc[t][j], 0, 0, 0);
-          }
-        }
-      }
+    for (int step = 0; step < steps; step += 2 * UNROLL) {
+      request(b1, kc + (step + UNROLL) * 32);               // past k_end a request loads nothing
+      multiply(b0, step, steps);
+      request(b0, kc + (step + 2 * UNROLL) * 32);           // may be the first group of the next chunk
+      multiply(b1, step + UNROLL, steps);
     }
   }
   // lane holds D[m = 4 kb + i][n = r] of each tile
@@ -114,9 +126,12 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
                          int chunk, hipStream_t s) {
   const int steps = (K + 31) / 32;
   const int steps_per_split = (steps + splits - 1) / splits;
+  const int grain = 64 * UNROLL;                                         // the k loop runs in pairs of UNROLL steps
   if (chunk <= 0 || chunk > steps_per_split * 32) chunk = steps_per_split * 32;
+  chunk = (chunk + grain - 1) / grain * grain;
   const size_t cap = 64 * 1024 / (16 * MT * sizeof(bf16_t));             // elements per row that fit 64 KB
-  if ((size_t)chunk + GEMM_LDS_PAD > cap) chunk = (int)((cap - GEMM_LDS_PAD) / 32 * 32);
+  if ((size_t)chunk + GEMM_LDS_PAD > cap) chunk = (int)((cap - GEMM_LDS_PAD) / grain * grain);
+  if (chunk < grain) return -1;
   const size_t lds = (size_t)16 * MT * (chunk + GEMM_LDS_PAD) * sizeof(bf16_t);
   dim3 grid((N + 128 * NT - 1) / (128 * NT), (M + 16 * MT - 1) / (16 * MT), splits);
   const bool aligned = (K % 8 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);

@@ -19,8 +19,8 @@ from . import library
 STREAM_GEMM_MAX_ROWS = 16
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
-# Blocks the matrix-core decode kernel aims for (256 CUs).
-DECODE_BLOCKS = 1024
+# Blocks the matrix-core decode kernel aims for (256 CUs; measured best at 8 rows x 2048 keys).
+DECODE_BLOCKS = 512
 
 
 class UnsupportedShape(ValueError):
@@ -164,12 +164,13 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
         _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _stream()), 'gemm_f32')
         return out
     _code(x.dtype)
-    if n <= STREAM_GEMM_MAX_ROWS and partials and bias is None and out_dtype == x.dtype:
+    streams = n <= STREAM_GEMM_MAX_ROWS
+    if streams and partials and bias is None and out_dtype == x.dtype:
         splits = lib.qil_gemm_bf16_splits(n, o, k)
         out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
         _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, 0, 0, _stream()), 'gemm_bf16')
         return Partials(out)
-    if out_dtype == torch.float32 or n <= STREAM_GEMM_MAX_ROWS:
+    if out_dtype == torch.float32 or streams:
         out = torch.empty((n, o), dtype=out_dtype, device=x.device)
         _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), 1, 0, 0,
                                  _stream()), 'gemm_bf16')
