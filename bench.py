@@ -54,6 +54,8 @@ def main():
     parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
     parser.add_argument('--points', default='1,64', help='other decode batch sizes to report, comma separated')
     parser.add_argument('--prefill-tokens', type=int, default=2048)
+    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill'],
+                        help='measure only one phase (for profiling); the JSON line then lacks the other')
     args = parser.parse_args()
     if args.gpus != 1:
         print(f'bench.py measures one GPU: this engine runs on a single MI355X (asked for {args.gpus})')
@@ -122,8 +124,15 @@ def main():
     def note(text):
         print(f'[bench] {text}', file=sys.stderr, flush=True)
 
+    if args.phase == 'prefill':
+        prefill_s = prefill_run(args.prefill_tokens)
+        print(json.dumps({'prefill_ms': round(prefill_s * 1e3, 3), 'tokens': args.prefill_tokens, 'layers': args.layers}))
+        return 0
     step_s, contexts = decode_run(args.batch)
     note(f'decode batch {args.batch}: {step_s * 1e3:.3f} ms/step')
+    if args.phase == 'decode':
+        print(json.dumps({'decode_ms_per_step': round(step_s * 1e3, 4), 'batch': args.batch, 'layers': args.layers}))
+        return 0
     points = {}
     for batch in [int(b) for b in args.points.split(',') if b]:
         seconds, _ = decode_run(batch)

@@ -138,6 +138,36 @@ def decoder_layer(x, weights, index, config, positions):
     return mlp_block(x, weights, prefix, config)
 
 
+def scheduled_hidden_states(tokens, weights, config, schedule):
+    """Hidden states when the layers run in the order of `schedule`, a list of (layer, cache_of):
+    a layer may run more than once, and an entry with cache_of = j attends over the keys and values
+    that entry j computed (from entry j's input) instead of its own.  Not in the reference, which runs
+    each layer once in order (qil/model.py:127-129); the parts are the reference's."""
+    tokens = torch.as_tensor(tokens, dtype=torch.long)
+    positions = torch.arange(len(tokens))
+    nq, nkv, d = config['num_attention_heads'], config['num_key_value_heads'], config['head_dim']
+    eps, theta = config.get('rms_norm_eps', 1e-6), config.get('rope_theta', 1000000.)
+    x = weights['model.embed_tokens.weight'][tokens]
+    kept = []
+    for layer, cache_of in schedule:
+        prefix = f'model.layers.{layer}.'
+        a = prefix + 'self_attn.'
+        n = rms_norm(x, weights[prefix + 'input_layernorm.weight'], eps)
+        T = x.shape[0]
+        angles = rotary_angles(positions, d, theta)
+        q = rotate(rms_norm(linear(n, weights[a + 'q_proj.weight']).reshape(T, nq, d), weights[a + 'q_norm.weight'], eps), angles)
+        if cache_of is None:
+            k = rotate(rms_norm(linear(n, weights[a + 'k_proj.weight']).reshape(T, nkv, d), weights[a + 'k_norm.weight'], eps), angles)
+            v = linear(n, weights[a + 'v_proj.weight']).reshape(T, nkv, d)
+        else:
+            k, v = kept[cache_of]
+        kept.append((k, v))
+        attended = attention(q, k, v, positions, d ** -0.5).reshape(T, nq * d)
+        x = x + linear(attended, weights[a + 'o_proj.weight'])
+        x = mlp_block(x, weights, prefix, config)
+    return x
+
+
 def head_weight(weights, config):
     """Tied head shares the embedding (default when the key is absent).
 
@@ -266,6 +296,12 @@ TINY_B = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size
               intermediate_size=224, num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=2,
               head_dim=32, max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=1000000.0,
               attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=[7, 9])
+
+# Sizes that are no multiple of 4 or 8 (the kernels' slow paths), an odd vocabulary, one head.
+TINY_D = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=131, hidden_size=50,
+              intermediate_size=70, num_hidden_layers=2, num_attention_heads=1, num_key_value_heads=1,
+              head_dim=64, max_position_embeddings=300, rms_norm_eps=2e-6, rope_theta=20000.0,
+              attention_bias=False, tie_word_embeddings=True, hidden_act='silu', eos_token_id=None)
 
 # A third variant: biases on q/k/v/o, sizes that are neither powers of two nor multiples of 32,
 # an odd vocabulary, MQA-like grouping.

@@ -14,7 +14,7 @@ import plain_qwen3 as plain
 from qil_amd.engine import ModelRunner, StepEntry
 from qil_amd.weights import load_model
 
-CONFIGS = {'A': (plain.TINY_A, 0, 4), 'B': (plain.TINY_B, 1, 8), 'C': (plain.TINY_C, 2, 3)}
+CONFIGS = {'A': (plain.TINY_A, 0, 4), 'B': (plain.TINY_B, 1, 8), 'C': (plain.TINY_C, 2, 3), 'D': (plain.TINY_D, 3, 16)}
 
 
 def poison(runner):
@@ -237,3 +237,33 @@ def test_graph_replays_equal_eager_launches(model_folder, dtype):
     expected = plain.logits(prompts['a'], weights, config)
     got = torch.cat([step[1:2] if step.shape[0] == 2 else step[0:1] for step in outputs[0]])[:8].cpu()
     torch.testing.assert_close(got, expected[5:13], **TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize('backend', BACKENDS, indirect=True)
+def test_schedule_with_a_repeated_layer_and_a_shared_cache(model_folder, backend):
+    """The run order is data: layer 0 runs twice (each run with a cache of its own) and the last entry
+    reads layer 1's cache instead of writing one.  Chunked steps equal the plain whole-sequence run."""
+    from qil_amd.parts import ScheduleEntry
+    from qil_amd.registry import read_model_config
+    from qil_amd.weights import load_weights
+    device, dtype = backend
+    config, seed, page_size = CONFIGS['B']
+    folder, weights = model_folder(config, seed)
+    entry, typed = read_model_config(folder)
+    model = entry.build(typed, dtype=dtype, device=device)
+    model.schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(2), ScheduleEntry(1, cache_of=1)]
+    load_weights(model, folder)
+    order = [(0, None), (1, None), (0, None), (2, None), (1, 1)]
+    tokens = tokens_for(config, 41, 17)
+    hidden = plain.scheduled_hidden_states(tokens, weights, config, order)
+    expected = plain.linear(plain.rms_norm(hidden, weights['model.norm.weight'], config['rms_norm_eps']),
+                            plain.head_weight(weights, config))
+    runner = ModelRunner(model, num_pages=8, page_size=page_size)
+    poison(runner)
+    assert runner.cache.kv_groups[0]['k'].shape[0] == 4           # four owning entries, one reader
+    runner.admit('r')
+    got, at = [], 0
+    for size in (9, 2, 17, 1, 1, 11):
+        got.append(runner.step([StepEntry('r', tuple(tokens[at:at + size]), tuple(range(size)))]))
+        at += size
+    Case(config, weights, model, page_size, dtype).close(torch.cat(got), expected)
