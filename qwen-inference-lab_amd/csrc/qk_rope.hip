@@ -85,6 +85,104 @@ __global__ void qk_norm_rope_store_kernel(
   }
 }
 
+// The same work with eight consecutive elements a lane (16-byte vectors) and no LDS: a head is spread
+// over TG = d / 8 lanes (a power of two), a wave serves 64 / TG (token, head) pairs, the statistics are
+// reduced and the rotation partner (TG lanes... rot / 16 lanes away) is fetched with lane shuffles.
+// Takes d in {16, 32, 64, 128, 256} and a rotated width whose half is a power-of-two number of
+// 8-element chunks (rot == d always qualifies).
+__device__ __forceinline__ void load8_sum(const float* base, size_t index, int splits, size_t stride, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 4) {
+    float4 lo[4], hi[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float* p = base + (size_t)min(s0 + u, splits - 1) * stride + index;
+      lo[u] = *reinterpret_cast<const float4*>(p);
+      hi[u] = *reinterpret_cast<const float4*>(p + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s0 + u < splits) {
+        out[0] += lo[u].x; out[1] += lo[u].y; out[2] += lo[u].z; out[3] += lo[u].w;
+        out[4] += hi[u].x; out[5] += hi[u].y; out[6] += hi[u].z; out[7] += hi[u].w;
+      }
+  }
+}
+__device__ __forceinline__ void load8_sum(const bf16_t* base, size_t index, int, size_t, float* out) { ld8(base + index, out); }
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+}
+
+template <typename TD, typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_vec_kernel(
+    const TD* __restrict__ qkv, int splits, size_t split_stride, T* __restrict__ q_out,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size,
+    float eps, int tg_log2) {
+  const int total_heads = heads + 2 * kv_heads;
+  const int TG = 1 << tg_log2;
+  const int pair = (int)((blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> tg_log2);    // (token, head) pair
+  const int chunk = threadIdx.x & (TG - 1);
+  if (pair >= n * total_heads) return;                  // whole lane groups leave together
+  const int token = pair / total_heads, head = pair - token * total_heads;
+  const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
+  if (!is_q && slots == nullptr) return;
+  float x[8];
+  load8_sum(qkv, ((size_t)token * total_heads + head) * d + chunk * 8, splits, split_stride, x);
+
+  if (!is_q && !is_k) {                                 // v: copy, transposed within the page
+    const int kvh = head - heads - kv_heads, slot = slots[token];
+    const size_t page = slot / page_size, offset = slot % page_size;
+    T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + chunk * 8) * page_size + offset;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) st(column + (size_t)e * page_size, x[e]);
+    return;
+  }
+  const float* weight = is_q ? q_weight : k_weight;
+  if (weight) {
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
+    for (int o = TG >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, QIL_WAVE);
+    const float rstd = rsqrtf(sum / (float)d + eps);
+    const float4 w0 = *reinterpret_cast<const float4*>(weight + chunk * 8);
+    const float4 w1 = *reinterpret_cast<const float4*>(weight + chunk * 8 + 4);
+    const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = round_to<T>(x[e] * rstd) * w[e];
+  }
+  if (cos_table && rot > 0) {
+    const int half_chunks = rot >> 4;                   // chunks in half of the rotated width (a power of two)
+    float other[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(x[e], half_chunks, QIL_WAVE);
+    if (chunk < 2 * half_chunks) {
+      const bool first = chunk < half_chunks;
+      const size_t at = (size_t)positions[token] * (rot >> 1) + (first ? chunk : chunk - half_chunks) * 8;
+      const float4 c0 = *reinterpret_cast<const float4*>(cos_table + at), c1 = *reinterpret_cast<const float4*>(cos_table + at + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(sin_table + at), s1 = *reinterpret_cast<const float4*>(sin_table + at + 4);
+      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = first ? x[e] * c[e] - other[e] * sn[e] : other[e] * sn[e] + x[e] * c[e];
+    }
+  }
+  if (is_q) {
+    store8(q_out + ((size_t)token * heads + head) * d + chunk * 8, x);
+  } else {
+    const int kvh = head - heads, slot = slots[token];
+    const size_t page = slot / page_size, offset = slot % page_size;
+    store8(k_cache + ((page * kv_heads + kvh) * page_size + offset) * (size_t)d + chunk * 8, x);
+  }
+}
+
 // qkv: in_dtype QIL_BF16 (one array, splits == 1) or QIL_F32 ([splits][n][..] partial sums).  dtype: type
 // of q_out and of the caches.
 extern "C" int qil_qk_norm_rope_store(
@@ -96,6 +194,27 @@ extern "C" int qil_qk_norm_rope_store(
   if (dtype == QIL_F32 && in_dtype != QIL_F32) return -1;
   const size_t stride = (size_t)n * (heads + 2 * kv_heads) * d;
   dim3 grid(n, heads + 2 * kv_heads);
+  // vector kernel: d / 8 a power of two up to 32, half of the rotated width a power-of-two number of chunks
+  int tg_log2 = -1;
+  for (int b = 1; b <= 5; ++b)
+    if (d == (8 << b)) tg_log2 = b;
+  const int half_chunks = rot >> 4;
+  const bool rot_fits = rot == 0 || !cos_table || (rot % 16 == 0 && (half_chunks & (half_chunks - 1)) == 0);
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)q_weight | (uintptr_t)k_weight |
+                         (uintptr_t)cos_table | (uintptr_t)sin_table) % 16) == 0;
+  if (tg_log2 > 0 && rot_fits && aligned) {
+    const size_t lanes = (size_t)n * (heads + 2 * kv_heads) << tg_log2;
+    const unsigned blocks = (unsigned)((lanes + 255) / 256);
+#define QIL_QKV_CASE(TD, T)                                                                                           \
+  hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)qkv, splits,    \
+                     stride, (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache,       \
+                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2)
+    if (dtype == QIL_F32) QIL_QKV_CASE(float, float);
+    else if (in_dtype == QIL_F32) QIL_QKV_CASE(float, bf16_t);
+    else QIL_QKV_CASE(bf16_t, bf16_t);
+#undef QIL_QKV_CASE
+    QIL_RETURN_LAUNCH_STATUS();
+  }
 #define QIL_QK_CASE(TD, T)                                                                                            \
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TD, T>), grid, dim3(QIL_WAVE), 0, s, (const TD*)qkv, splits, stride,   \
                      (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache, (T*)v_cache,  \
