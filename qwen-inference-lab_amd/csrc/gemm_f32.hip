@@ -1,10 +1,11 @@
 // True float32 matrix product for the 32-bit path: C[M, N] = A[M, K] W[N, K]^T (+ bias[N]).
 //
-// Inputs, products and sums are IEEE float32 FMA on the vector units: no matrix-core mode, no
-// reduced-precision inputs, no split of K across threads, so every element of C is one thread's
-// sequential sum over k and does not depend on M, on the row's place in the batch or on the tile
-// it falls into.  Both operands have K contiguous (nn.Linear layout, qil/model.py:32-40).
-// 64 x 64 x 16 tiles in LDS, 256 threads, 4 x 4 outputs a thread.
+// Many rows: inputs, products and sums are IEEE float32 FMA on the vector units, no split of K
+// across threads, so every element of C is one thread's sequential sum over k and does not depend
+// on M, on the row's place in the batch or on the tile it falls into.  Few rows: see the streaming
+// kernel below (float32 matrix-core instruction, still no reduced-precision input).  Both operands
+// have K contiguous (nn.Linear layout, qil/model.py:32-40).  The tiled kernel: 64 x 64 x 16 tiles in
+// LDS, 256 threads, 4 x 4 outputs a thread.
 #include "common.h"
 
 #define SG_BM 64
@@ -105,10 +106,107 @@ sgemv_rows_kernel(const float* __restrict__ A, const float* __restrict__ W, cons
   }
 }
 
+// Few rows (decode), K % 4 == 0: the product is bound by streaming W once, so it is shaped like the
+// bfloat16 streaming kernel (gemm_bf16.hip): a block owns 128 columns (8 waves x 16) and one of
+// `splits` ranges of K, stages its slice of A in LDS, and every wave streams its 16 rows of W from
+// global memory straight into v_mfma_f32_16x16x4_f32 operands: float32 inputs, float32 products and
+// sums on the matrix cores (no reduced-precision mode exists for this instruction).  A lane's
+// float4 of W (row r, columns 4 kb .. 4 kb + 3 of a 16-column step) feeds four products, A's float4
+// from LDS being laid out the same way.  With splits > 1 the block writes a partial result
+// C[split, M, N] that the consuming kernel adds in split order.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+#define SF_WAVES 8
+#define SF_PAD 4
+
+template <int MT, int UNROLL>
+__global__ void __launch_bounds__(SF_WAVES * QIL_WAVE)
+gemm_f32_stream_kernel(const float* __restrict__ A, const float* __restrict__ W, const float* __restrict__ bias,
+                       float* __restrict__ C, int M, int N, int K, int steps_per_split, int chunk) {
+  extern __shared__ __align__(16) float a_lds[];           // [16 MT][chunk + pad]
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int n0 = (blockIdx.x * SF_WAVES + wave) * 16, m0 = blockIdx.y * 16 * MT, split = blockIdx.z;
+  const int row_width = chunk + SF_PAD;
+  f32x4v acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+  const int k_begin = split * steps_per_split * 16, k_end = min(K, k_begin + steps_per_split * 16);
+  const bool row_live = n0 + r < N;
+  const float* w_row = W + (size_t)(row_live ? n0 + r : 0) * K;
+  for (int kc = k_begin; kc < k_end; kc += chunk) {
+    const int width = min(chunk, k_end - kc);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 16 * MT * (chunk / 4); idx += SF_WAVES * QIL_WAVE) {
+      const int m = idx / (chunk / 4), c = (idx - m * (chunk / 4)) * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < width && m0 + m < M) v = *reinterpret_cast<const float4*>(A + (size_t)(m0 + m) * K + kc + c);
+      *reinterpret_cast<float4*>(a_lds + m * row_width + c) = v;
+    }
+    __syncthreads();
+    const int steps = (width + 15) / 16;
+    for (int step = 0; step < steps; step += UNROLL) {
+      float4 b[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int k = kc + (step + u) * 16 + kb * 4;
+        b[u] = (step + u < steps && row_live && k < k_end) ? *reinterpret_cast<const float4*>(w_row + k)
+                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if (step + u < steps) {
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const float4 a = *reinterpret_cast<const float4*>(a_lds + (t * 16 + r) * row_width + (step + u) * 16 + kb * 4);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b[u].x, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b[u].y, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b[u].z, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b[u].w, acc[t], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  float* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + t * 16 + 4 * kb + i, n = n0 + r;
+      if (m < M && n < N) out[(size_t)m * N + n] = acc[t][i] + (bias ? bias[n] : 0.f);
+    }
+}
+
+// Ways the few-row product will be split over K when partial sums are allowed (1: it is not split).
+extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
+  if (M > 16 || K % 4) return 1;
+  const int column_blocks = (N + 127) / 128, steps = (K + 15) / 16;
+  int sp = (768 + column_blocks - 1) / column_blocks;
+  if (sp > 8) sp = 8;
+  while (sp > 1 && steps / sp < 16) --sp;
+  return sp < 1 ? 1 : sp;
+}
+
+// C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs M <= 16,
+// K % 4 == 0 and no bias.
 extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
-                            hipStream_t s) {
+                            int splits, hipStream_t s) {
   if (M == 0 || N == 0) return 0;
-  if (K < 1) return -1;
+  if (K < 1 || splits < 1) return -1;
+  const bool stream_ok = M <= 16 && K % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+  if (splits > 1 && (!stream_ok || bias)) return -1;
+  if (stream_ok) {
+    const int steps = (K + 15) / 16, steps_per_split = (steps + splits - 1) / splits;
+    int chunk = steps_per_split * 16;
+    const int cap = (64 * 1024 / (16 * (int)sizeof(float)) - SF_PAD) / 64 * 64;      // columns per row within 64 KB
+    if (chunk > cap) chunk = cap;
+    chunk = (chunk + 15) / 16 * 16;
+    const size_t lds = (size_t)16 * (chunk + SF_PAD) * sizeof(float);
+    dim3 grid((N + 127) / 128, 1, splits);
+    hipLaunchKernelGGL((gemm_f32_stream_kernel<1, 4>), grid, dim3(SF_WAVES * QIL_WAVE), lds, s, A, W, bias, C, M, N, K,
+                       steps_per_split, chunk);
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   if (M <= 2 * SV_ROWS) {
     const int waves = 4;
     for (int m0 = 0; m0 < M; m0 += SV_ROWS)

@@ -160,9 +160,10 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     if x.dtype == torch.float32:
         if out_dtype != torch.float32:
             raise UnsupportedShape('a float32 product has a float32 result')
-        out = torch.empty((n, o), dtype=torch.float32, device=x.device)
-        _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _stream()), 'gemm_f32')
-        return out
+        splits = lib.qil_gemm_f32_splits(n, o, k) if partials and bias is None else 1
+        out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+        _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, splits, _stream()), 'gemm_f32')
+        return Partials(out) if splits > 1 else out[0]
     _code(x.dtype)
     streams = n <= STREAM_GEMM_MAX_ROWS
     if streams and partials and bias is None and out_dtype == x.dtype:
