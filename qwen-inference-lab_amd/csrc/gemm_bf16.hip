@@ -19,6 +19,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_out(bf16_t* p, float v) { *p = f32_to_bf16(v); }
@@ -144,6 +145,127 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
   return 0;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same product with W read in whole cache lines.  The fragment layout above makes every load
+// instruction touch 16 rows x 64 bytes; here a load instruction takes 4 rows x 256 contiguous bytes
+// (lane l: row 4 u + l / 16, 16-byte piece l % 16), three stages of 16 rows x 128 columns are in
+// flight in registers, and a stage passes through a wave-private 4 KB LDS buffer that turns it into
+// fragments.  The 16-byte pieces of a row are stored at piece ^ row, so the writes (16 lanes, one
+// row) and the fragment reads (16 lanes, 16 rows, one logical piece) both spread over all banks.
+// LDS operations of one wave complete in program order, so the buffer needs no barrier.
+// Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
+#define LINES_WAVES 8
+#define LINES_DEPTH 3                                      // stages of W in flight per wave
+#define LINES_LDS_LIMIT (80 * 1024)                        // two blocks on a CU's 160 KB
+
+template <typename OUT>
+__global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
+gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N,
+                       int K, int cols_per_split) {
+  extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
+  const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
+  const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
+  const int row_width = cols_per_split + GEMM_LDS_PAD;
+  bf16_t* a_lds = lds;
+  bf16_t* buffer = lds + a_rows * row_width + wave * (16 * 128);
+
+  const int load_row = lane >> 4, piece = lane & 15;
+  const bf16_t* source[4];                                 // rows past N read a valid row and are never stored
+  int place[4];                                            // where this lane's piece of load u goes in the buffer
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    source[u] = W + (size_t)min(n0 + row, N - 1) * K + k_begin + piece * 8;
+    place[u] = row * 128 + ((piece ^ row) & 15) * 8;
+  }
+  // A slice first: its wait would otherwise cover the first stages of W as well
+  for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
+    const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (m < M) v = *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
+    *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+  }
+  // three stages in flight, each in registers of its own (named, so that none is indexed at run time)
+  u32x4 w0[4], w1[4], w2[4];
+  auto request = [&](u32x4 (&stage_w)[4], int stage) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const u32x4*>(source[u] + stage * 128);
+  };
+  request(w0, 0);                                           // the host sees to stages >= 3
+  request(w1, 1);
+  request(w2, 2);
+  __syncthreads();
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bool a_live = r < a_rows;
+  const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + kb * 8;
+  auto pass = [&](const u32x4 (&stage_w)[4]) {             // registers -> buffer
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = stage_w[u];
+  };
+  auto multiply = [&](int stage) {
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
+      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + stage * 128 + s4 * 32);
+      if (!a_live) a = (u32x4){0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
+                                                    0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  int stage = 0;
+  for (; stage + 6 <= stages; stage += 3) {                 // every stage here has a successor three ahead
+    pass(w0); request(w0, stage + 3); multiply(stage);
+    pass(w1); request(w1, stage + 4); multiply(stage + 1);
+    pass(w2); request(w2, stage + 5); multiply(stage + 2);
+  }
+  // the last three to five stages: requests run out
+  const int left = stages - stage;
+  pass(w0); if (left > 3) request(w0, stage + 3); multiply(stage);
+  pass(w1); if (left > 4) request(w1, stage + 4); multiply(stage + 1);
+  pass(w2); multiply(stage + 2);
+  if (left > 3) { pass(w0); multiply(stage + 3); }
+  if (left > 4) { pass(w1); multiply(stage + 4); }
+  OUT* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = 4 * kb + i, n = n0 + r;
+    if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[i]);
+  }
+}
+
+static size_t lines_lds(int M, int K, int splits) {
+  return ((size_t)(M <= 8 ? 8 : 16) * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
+}
+
+// Whether the whole-line kernel takes the product with this many splits.
+static bool lines_takes(const void* A, const void* W, const float* bias, int M, int N, int K, int splits) {
+  if (bias || M > 16 || N < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH ||
+      (((uintptr_t)A | (uintptr_t)W) % 16))
+    return false;
+  return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
+}
+
+template <typename OUT>
+static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
+  const size_t lds = lines_lds(M, K, splits);
+  auto kernel = gemm_bf16_lines_kernel<OUT>;
+  static size_t granted = 0;                              // per instantiation
+  if (lds > 64 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
+  return 0;
+}
+
 // Shapes of the kernel that exist: code = MT * 100 + NT * 10 + UNROLL.
 #define QIL_GEMM_SHAPES(X) \
   X(1, 1, 4) X(1, 1, 8) X(1, 2, 4) X(1, 2, 8) X(1, 4, 4) X(2, 1, 4) X(2, 1, 8) X(2, 2, 4) X(4, 1, 4) X(4, 1, 8) \
@@ -192,6 +314,16 @@ extern "C" int qil_gemm_bf16(const void* A, const void* W, const float* bias, vo
   if (M == 0 || N == 0) return 0;
   if (K < 1 || splits < 1 || splits > 65535 || (splits > 1 && (out_dtype != QIL_F32 || bias))) return -1;
   int code = shape, planned;
+  if (code == 0 || code == 1) {                              // 1: force the whole-line kernel (tuning runs)
+    if (lines_takes(A, W, bias, M, N, K, splits)) {
+      const int status = out_dtype == QIL_F32
+                             ? launch_lines<float>((const bf16_t*)A, (const bf16_t*)W, (float*)C, M, N, K, splits, s)
+                             : launch_lines<bf16_t>((const bf16_t*)A, (const bf16_t*)W, (bf16_t*)C, M, N, K, splits, s);
+      if (status) return status;
+      QIL_RETURN_LAUNCH_STATUS();
+    }
+    if (code == 1) return -1;
+  }
   if (!code) plan(M, N, K, false, &code, &planned);
   int status;
   if (out_dtype == QIL_F32)
