@@ -188,11 +188,16 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
     if (m < M) v = *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
     *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
   }
+  // Every wave walks its K range from a start of its own and wraps around: waves that all read the
+  // same columns of their rows at the same time load a few memory channels only.
+  const int turn = (n0 / 16) % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * 128; };
   // three stages in flight, each in registers of its own (named, so that none is indexed at run time)
   u32x4 w0[4], w1[4], w2[4];
   auto request = [&](u32x4 (&stage_w)[4], int stage) {
+    const int at = column(stage);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const u32x4*>(source[u] + stage * 128);
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const u32x4*>(source[u] + at);
   };
   request(w0, 0);                                           // the host sees to stages >= 3
   request(w1, 1);
@@ -207,11 +212,12 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
     for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = stage_w[u];
   };
   auto multiply = [&](int stage) {
+    const int at = column(stage);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
-      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + stage * 128 + s4 * 32);
+      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
       if (!a_live) a = (u32x4){0, 0, 0, 0};
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
                                                     0, 0);
@@ -264,6 +270,191 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
   dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
   hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Gate and up products of a gated feed-forward with the activation in the epilogue:
+//   out[m, n] = silu(A W[n]^T) * (A W[inner + n]^T),  n < inner        (qil/model.py:71)
+// W is the stacked [2 inner, K] matrix, gate rows first.  A "pair" is 16 gate rows and the 16 up rows
+// that belong to them.  A block owns `pairs` consecutive pairs and `ksplit` waves per pair, which split
+// K among themselves and add their float32 sums in LDS in wave order, so nothing but the finished
+// activations leaves the block: no partial sums in memory and no separate activation pass.  All of A
+// (8 or 16 rows) sits in LDS once per block.  W is read in whole cache lines as in the kernel above
+// (two stages in flight, gate and up taking turns in the wave's buffer).
+// Takes M <= 16 (while A fits in LDS), inner a multiple of 16, K a multiple of 128 ksplit with at least 2 stages a wave,
+// 16-byte aligned operands.
+#define GATED_MAX_WAVES 12                                 // three waves a SIMD: 168 registers each
+
+template <typename OUT>
+__global__ void __launch_bounds__(GATED_MAX_WAVES * QIL_WAVE)
+gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ out, int M,
+                       int inner, int K, int ksplit) {
+  extern __shared__ __align__(16) bf16_t lds[];            // A [8 or 16][K + pad], then a 4 KB buffer per wave
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int pair = wave / ksplit, part = wave - pair * ksplit;
+  const int pairs = blockDim.x / QIL_WAVE / ksplit;
+  // a pair past the end repeats the last one and stores nothing
+  const int n0 = min(blockIdx.x * pairs + pair, inner / 16 - 1) * 16;
+  const bool stores = (blockIdx.x * pairs + pair) * 16 < inner;
+  const int cols_per_wave = K / ksplit, k_begin = part * cols_per_wave, stages = cols_per_wave / 128;
+  const int row_width = K + GEMM_LDS_PAD;
+  bf16_t* a_lds = lds;
+  bf16_t* buffer = lds + a_rows * row_width + wave * (16 * 128);
+
+  // this lane's part of a stage: rows 4 u + lane / 16 (u < 4), 16-byte piece lane % 16, stored at piece ^ row
+  const int load_row = lane >> 4, piece = lane & 15;
+  const bf16_t* gate_source[4];
+  int place[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    gate_source[u] = W + (size_t)(n0 + row) * K + k_begin + piece * 8;
+    place[u] = row * 128 + ((piece ^ row) & 15) * 8;
+  }
+  const size_t up_offset = (size_t)inner * K;
+  // Every wave walks its K range from a start of its own and wraps around: waves that all read the
+  // same columns of their rows at the same time load a few memory channels only.
+  const int turn = (n0 / 16) % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * 128; };
+
+  u32x4 g0[4], u0[4], g1[4], u1[4];                        // two stages, named so that none is indexed at run time
+  auto request = [&](u32x4 (&w)[4], size_t offset, int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) w[u] = *reinterpret_cast<const u32x4*>(gate_source[u] + offset + at);
+  };
+  // A first (its wait would otherwise cover W's first stages), then W's first two stages
+  for (int idx = threadIdx.x; idx < a_rows * (K / 8); idx += blockDim.x) {
+    const int m = idx / (K / 8), c = (idx - m * (K / 8)) * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (m < M) v = *reinterpret_cast<const uint4*>(A + (size_t)m * K + c);
+    *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+  }
+  request(g0, 0, 0); request(u0, up_offset, 0);             // the host sees to stages >= 2
+  request(g1, 0, 1); request(u1, up_offset, 1);
+  __syncthreads();
+
+  f32x4 gate = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
+  const bool a_live = r < a_rows;
+  const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + k_begin + kb * 8;
+  auto pass = [&](const u32x4 (&w)[4]) {                   // registers -> buffer
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = w[u];
+  };
+  auto multiply = [&](int stage, f32x4& acc) {
+    const int at = column(stage);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
+      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
+      if (!a_live) a = (u32x4){0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
+                                                    0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  int stage = 0;
+  for (; stage + 4 <= stages; stage += 2) {                 // both stages here have a successor two ahead
+    pass(g0); request(g0, 0, stage + 2); multiply(stage, gate);
+    pass(u0); request(u0, up_offset, stage + 2); multiply(stage, up);
+    pass(g1); request(g1, 0, stage + 3); multiply(stage + 1, gate);
+    pass(u1); request(u1, up_offset, stage + 3); multiply(stage + 1, up);
+  }
+  const bool three = stages - stage == 3;                   // two or three stages are left
+  pass(g0); if (three) request(g0, 0, stage + 2);
+  multiply(stage, gate);
+  pass(u0); if (three) request(u0, up_offset, stage + 2);
+  multiply(stage, up);
+  pass(g1); multiply(stage + 1, gate);
+  pass(u1); multiply(stage + 1, up);
+  if (three) {
+    pass(g0); multiply(stage + 2, gate);
+    pass(u0); multiply(stage + 2, up);
+  }
+
+  // the waves' sums meet in LDS (in the buffers, which every wave has finished with): [wave][gate, up][lane][4]
+  __syncthreads();
+  float* sums = reinterpret_cast<float*>(lds + a_rows * row_width);
+  *reinterpret_cast<f32x4*>(sums + ((wave * 2 + 0) * QIL_WAVE + lane) * 4) = gate;
+  *reinterpret_cast<f32x4*>(sums + ((wave * 2 + 1) * QIL_WAVE + lane) * 4) = up;
+  __syncthreads();
+  if (part == 0 && stores) {
+    f32x4 g = {0.f, 0.f, 0.f, 0.f}, v = {0.f, 0.f, 0.f, 0.f};
+    for (int w = wave; w < wave + ksplit; ++w) {            // fixed order
+      g += *reinterpret_cast<const f32x4*>(sums + ((w * 2 + 0) * QIL_WAVE + lane) * 4);
+      v += *reinterpret_cast<const f32x4*>(sums + ((w * 2 + 1) * QIL_WAVE + lane) * 4);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * kb + i, n = n0 + r;                 // lane holds D[m = 4 kb + i][n = r]
+      if (m < M) store_out(out + (size_t)m * inner + n, (g[i] / (1.f + expf(-g[i]))) * v[i]);
+    }
+  }
+}
+
+// The block shape of the gated kernel for these sizes (pairs a block, waves a pair); false if it does
+// not take them.
+static size_t gated_lds(int M, int K, int waves) {
+  return ((size_t)(M <= 8 ? 8 : 16) * (K + GEMM_LDS_PAD) + (size_t)waves * 16 * 128) * sizeof(bf16_t);
+}
+
+static bool gated_plan(const void* A, const void* W, int M, int inner, int K, int* pairs, int* ksplit) {
+  if (M < 1 || M > 16 || inner < 16 || inner % 16 || K % 128 || (((uintptr_t)A | (uintptr_t)W) % 16))
+    return false;
+  int ks = 0;
+  for (int c = 8; c >= 1 && !ks; c /= 2)                   // most waves that still leave 16 stages each; else 2 stages
+    if (K % (128 * c) == 0 && K / (128 * c) >= (c == 1 ? 2 : 16)) ks = c;
+  if (!ks) return false;
+  const int all_pairs = inner / 16;
+  int best = 0;
+  long best_cost = 0;
+  for (int pb = GATED_MAX_WAVES / ks; pb >= 1; --pb) {      // rounds of 256 CUs x pairs a block; ties go to more pairs
+    if (gated_lds(M, K, pb * ks) > 156 * 1024) continue;
+    const long blocks = (all_pairs + pb - 1) / pb, cost = (blocks + 255) / 256 * pb;
+    if (!best || cost < best_cost) { best = pb; best_cost = cost; }
+  }
+  if (!best) return false;
+  *pairs = best;
+  *ksplit = ks;
+  return true;
+}
+
+extern "C" int qil_gemm_bf16_gated_takes(int M, int inner, int K) {
+  int pairs, ksplit;
+  return gated_plan(nullptr, nullptr, M, inner, K, &pairs, &ksplit);
+}
+
+// out [M, inner] of out_dtype = silu(A W[:inner]^T) * (A W[inner:]^T).  pairs, ksplit: 0 = chosen here
+// (tuning runs set them).
+extern "C" int qil_gemm_bf16_gated(const void* A, const void* W, void* out, int M, int inner, int K, int out_dtype,
+                                   int pairs, int ksplit, hipStream_t s) {
+  if (M == 0 || inner == 0) return 0;
+  int planned_pairs, planned_ksplit;
+  if (!gated_plan(A, W, M, inner, K, &planned_pairs, &planned_ksplit)) return -1;
+  if (!pairs) pairs = planned_pairs;
+  if (!ksplit) ksplit = planned_ksplit;
+  if (pairs < 1 || ksplit < 1 || pairs * ksplit > GATED_MAX_WAVES || K % (128 * ksplit) || K / (128 * ksplit) < 2) return -1;
+  const size_t lds = gated_lds(M, K, pairs * ksplit);
+  if (lds > 160 * 1024) return -1;
+  const int all_pairs = inner / 16;
+  dim3 grid((all_pairs + pairs - 1) / pairs), block(pairs * ksplit * QIL_WAVE);
+#define QIL_GATED_CASE(OUT)                                                                                          \
+  {                                                                                                                  \
+    auto kernel = gemm_bf16_gated_kernel<OUT>;                                                                       \
+    static size_t granted = 0;                                                                                       \
+    if (lds > 64 * 1024 && lds > granted) {                                                                          \
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                                            \
+      granted = lds;                                                                                                 \
+    }                                                                                                                \
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)out, M, inner, K, ksplit); \
+  }
+  if (out_dtype == QIL_F32) QIL_GATED_CASE(float) else QIL_GATED_CASE(bf16_t)
+#undef QIL_GATED_CASE
+  QIL_RETURN_LAUNCH_STATUS();
 }
 
 // Shapes of the kernel that exist: code = MT * 100 + NT * 10 + UNROLL.

@@ -182,6 +182,27 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     return out
 
 
+def gated_linear(x, weight, out_dtype=None):
+    """silu(x @ gate^T) * (x @ up^T) with ``weight`` the stacked [2 I, K] matrix, gate rows first -> [N, I].
+
+    One kernel when the fused few-row kernel takes the sizes (bfloat16, at most 16 rows); otherwise the
+    product followed by ``silu_mul``.  Both add in float32 and round once."""
+    _require(x, 'x')
+    _require(weight, 'weight', x.dtype)
+    n, k = x.shape
+    both = weight.shape[0]
+    if weight.shape[1] != k or both % 2:
+        raise ValueError(f'gated_linear: x {tuple(x.shape)}, weight {tuple(weight.shape)}')
+    out_dtype = out_dtype or x.dtype
+    lib = library.load()
+    if x.dtype == torch.bfloat16 and n and lib.qil_gemm_bf16_gated_takes(n, both // 2, k):
+        out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
+        _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
+                                       _stream()), 'gemm_bf16_gated')
+        return out
+    return silu_mul(linear(x, weight, None, partials=True), out_dtype)
+
+
 def silu_mul(gate_up, out_dtype=None):
     """[N, 2 I] (gate columns first; tensor of the model's type or Partials) -> silu(gate) * up, [N, I]."""
     n, both = gate_up.shape

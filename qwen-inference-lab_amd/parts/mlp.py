@@ -27,5 +27,5 @@ class GatedMLP(FeedForward):
         p['gate_up_proj.weight'] = torch.cat([p.pop('gate_proj.weight'), p.pop('up_proj.weight')]).contiguous()
 
     def forward(self, h):
-        gate_up = ops.linear(h, self.p['gate_up_proj.weight'], None, partials=True)
-        return ops.linear(ops.silu_mul(gate_up, self.dtype), self.p['down_proj.weight'], None, partials=True)
+        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype)
+        return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

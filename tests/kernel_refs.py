@@ -46,6 +46,13 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     return y.to(out_dtype or x.dtype)
 
 
+def gated_linear(x, weight, out_dtype=None):
+    y = x.to(torch.float32) @ weight.to(torch.float32).t()
+    inner = y.shape[1] // 2
+    g, u = y[:, :inner], y[:, inner:]
+    return (g / (1 + torch.exp(-g)) * u).to(out_dtype or x.dtype)
+
+
 def silu_mul(gate_up, out_dtype=None):
     gate_up = _value(gate_up)
     inner = gate_up.shape[1] // 2
@@ -130,5 +137,5 @@ def sample(logits, temperatures, seeds, counters):
     return scores.argmax(dim=-1).to(torch.int32), finite
 
 
-ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, silu_mul=silu_mul,
+ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
            qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample)

@@ -139,11 +139,15 @@ def test_linear_partial_sums(ops, m, n, k):
 
 
 def test_linear_rows_do_not_depend_on_the_batch(ops):
-    """A row's result is the same alone, among 7 and among 40 (same kernel family): bit for bit."""
+    """A row's result is the same alone, among 7 and among 16 (one kernel, one order of the sums): bit for bit.
+    Among 40 another kernel adds the same exact products in another order: equal up to float32 rounding."""
     x, w = rand(40, 512, dtype=torch.bfloat16), rand(300, 512, dtype=torch.bfloat16, seed=1, scale=0.05)
+    few = ops.linear(x[:16].contiguous(), w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(ops.linear(x[3:4].contiguous(), w, None, out_dtype=torch.float32), few[3:4], atol=0, rtol=0)
+    torch.testing.assert_close(ops.linear(x[:7].contiguous(), w, None, out_dtype=torch.float32), few[:7], atol=0, rtol=0)
     whole = ops.linear(x, w, None, out_dtype=torch.float32)
-    torch.testing.assert_close(ops.linear(x[3:4].contiguous(), w, None, out_dtype=torch.float32), whole[3:4], atol=0, rtol=0)
-    torch.testing.assert_close(ops.linear(x[:7].contiguous(), w, None, out_dtype=torch.float32), whole[:7], atol=0, rtol=0)
+    torch.testing.assert_close(ops.linear(x[17:40].contiguous(), w, None, out_dtype=torch.float32), whole[17:], atol=0, rtol=0)
+    check(whole[:16], few.double(), torch.float32, scale=8)
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
@@ -155,6 +159,37 @@ def test_silu_mul(ops, dtype):
     total = parts[0] + parts[1] + parts[2]
     want = torch.nn.functional.silu(total[:, :136].double()) * total[:, 136:].double()
     check(ops.silu_mul(ops.Partials(parts), dtype), want, dtype, scale=8)
+
+
+@pytest.mark.parametrize('m,inner,k', [(1, 12288, 4096), (8, 3072, 1024), (5, 48, 384), (8, 208, 2048), (3, 16, 128),
+                                       (8, 1040, 256), (7, 136, 100), (12, 256, 1024), (40, 64, 256)])
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_gated_linear(ops, m, inner, k, dtype):
+    """silu(x gate^T) * (x up^T): the fused few-row kernel where it takes the sizes (rows <= 16, inner % 16 == 0,
+    K % 128 == 0), the product followed by the activation elsewhere; both against float64."""
+    x = rand(m, k, dtype=dtype)
+    w = rand(2 * inner, k, dtype=dtype, seed=1, scale=2.0 * k ** -0.5)
+    y = x.double() @ w.double().t()
+    want = torch.nn.functional.silu(y[:, :inner]) * y[:, inner:]
+    got = ops.gated_linear(x, w)
+    assert got.dtype == dtype and got.shape == (m, inner)
+    check(got, want, dtype, scale=8)
+
+
+def test_gated_linear_block_shapes(ops):
+    """Every block shape of the fused kernel (pairs a block x waves a pair) gives the same sums up to their order."""
+    from qil_amd.ops import library
+    lib = library.load()
+    m, inner, k = 8, 400, 2048
+    x = rand(m, k, dtype=torch.bfloat16)
+    w = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
+    y = x.double() @ w.double().t()
+    want = torch.nn.functional.silu(y[:, :inner]) * y[:, inner:]
+    stream = torch.cuda.current_stream().cuda_stream
+    for pairs, ksplit in ((1, 1), (3, 4), (12, 1), (1, 8), (2, 2), (5, 2), (6, 2)):
+        out = torch.full((m, inner), float('nan'), dtype=torch.float32, device='cuda')
+        assert lib.qil_gemm_bf16_gated(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, inner, k, 0, pairs, ksplit, stream) == 0
+        check(out, want, torch.float32, scale=8)
 
 
 class Rot:
