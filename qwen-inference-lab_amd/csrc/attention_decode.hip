@@ -9,26 +9,26 @@
 //   O^T[dim, head] = sum_key V^T[dim, key] P^T[key, head] A = V^T rows    (V is [.., d, page_size])
 //
 // The 16 columns of a tile are the g query heads of the kv head (columns from g on are zero), so
-// a lane holds the scores of ONE head for keys 4 (lane / 16) + i, and softmax statistics are
+// a lane holds the scores of ONE head for eight keys (8 (lane / 16) + j of a 32-key step: the rows
+// of the two 16-key score tiles are assigned to keys accordingly), and softmax statistics are
 // per-lane scalars reduced over the 4 lane groups by two shuffles (qil/paged_attention.py:27-41
-// computes the same maxima, sums and weighted values in float32).  Each of the block's 4 waves
-// takes every fourth 32-key step and keeps its own running (m, l, O); the four meet in LDS once.
+// computes the same maxima, sums and weighted values in float32).  Each of the block's waves
+// takes every waves-th 32-key step and keeps its own running (m, l, O); they meet in LDS once.
 //
 // Invisible keys (j > position, or outside the window) may lie in pages that were never
 // written or belong to someone else: their scores are replaced, not multiplied, and their V
 // elements are zeroed before the product, so garbage (even NaN) cannot enter a sum.
 //
-// Takes page_size % 4 == 0, d % 16 == 0, d <= 256, g <= 16; other sizes go to the row kernel.
+// Takes page_size % 8 == 0, d % 16 == 0, d <= 256, g <= 16; other sizes go to the row kernel.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define DEC_THREADS 256
-#define DEC_WAVES 4
+#define DEC_MAX_WAVES 8                                    // waves of a block; each takes every waves-th 32-key step
 
 template <int DMAX>
-__global__ void __launch_bounds__(DEC_THREADS)
+__global__ void __launch_bounds__(DEC_MAX_WAVES * QIL_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                    const int* __restrict__ row_seq, const int* __restrict__ positions,
@@ -45,7 +45,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   const int begin = max(part * P, lo), end = min((part + 1) * P, ctx);
   if (begin >= end) return;
 
-  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE, waves = blockDim.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
   const int dt = d / 16;
   const int* table = block_tables + (size_t)row_seq[row] * table_stride;
@@ -67,13 +67,15 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 
   const int first_step = begin / 32;                       // 32-key steps, absolute numbering
   const int last_step = (end - 1) / 32;
-  for (int step = first_step + wave; step <= last_step; step += DEC_WAVES) {
+  for (int step = first_step + wave; step <= last_step; step += waves) {
     const int k0 = step * 32;
     // ---- loads first: K rows of both 16-key sub-tiles, then the V^T fragments of every dim tile
     uint4 kraw[2][QFRAGS];
 #pragma unroll
     for (int jt = 0; jt < 2; ++jt) {
-      const int key = min(k0 + jt * 16 + r, ctx - 1);      // clamped: an invisible key's score is replaced below
+      // row r of sub-tile jt is key 8 (r / 4) + 4 jt + r % 4 of the step, so that a lane's eight
+      // scores (rows 4 kb + i of both sub-tiles) are the eight consecutive keys 8 kb .. 8 kb + 7
+      const int key = min(k0 + 8 * (r >> 2) + 4 * jt + (r & 3), ctx - 1);   // clamped: an invisible key's score is replaced below
       const size_t page = table[key / page_size];
       const bf16_t* krow = k_cache + ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d;
 #pragma unroll
@@ -82,21 +84,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
         kraw[jt][ks] = (ks * 32 < d && dim < d) ? *reinterpret_cast<const uint4*>(krow + dim) : make_uint4(0, 0, 0, 0);
       }
     }
-    uint2 vraw[DTILES][2];
+    uint4 vraw[DTILES];                                     // V^T[dim 16 t + r][keys 8 kb .. 8 kb + 7]: 16 bytes of one page row
     {
-      const bf16_t* vbase[2];
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const int key = min(k0 + hf * 16 + 4 * kb, ctx - 1) & ~3;    // group of 4 keys inside one page
-        const size_t page = table[key / page_size];
-        vbase[hf] = v_cache + (page * kv_heads + kvh) * (size_t)d * page_size + (key % page_size);
-      }
+      const int key = min(k0 + 8 * kb, ctx - 1) & ~7;
+      const size_t page = table[key / page_size];
+      const bf16_t* vbase = v_cache + (page * kv_heads + kvh) * (size_t)d * page_size + (key % page_size);
 #pragma unroll
       for (int t = 0; t < DTILES; ++t)
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-          vraw[t][hf] = t < dt ? *reinterpret_cast<const uint2*>(vbase[hf] + (size_t)(t * 16 + r) * page_size)
-                               : make_uint2(0, 0);
+        vraw[t] = t < dt ? *reinterpret_cast<const uint4*>(vbase + (size_t)(t * 16 + r) * page_size) : make_uint4(0, 0, 0, 0);
     }
     // ---- scores
     f32x4 s[2];
@@ -114,7 +109,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = k0 + jt * 16 + 4 * kb + i;
+        const int key = k0 + 8 * kb + 4 * jt + i;
         const bool visible = key >= begin && key < end;
         keep[jt][i] = visible ? 0xffffu : 0u;
         const float v = visible ? s[jt][i] * scale : -INFINITY;
@@ -149,8 +144,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 #pragma unroll
     for (int t = 0; t < DTILES; ++t) {
       if (t < dt) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vraw[t][0].x & mask[0], vraw[t][0].y & mask[1],
-                                                                vraw[t][1].x & mask[2], vraw[t][1].y & mask[3]));
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vraw[t].x & mask[0], vraw[t].y & mask[1],
+                                                                vraw[t].z & mask[2], vraw[t].w & mask[3]));
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
         o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[t], 0, 0, 0);
@@ -158,7 +153,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     }
   }
 
-  // ---- the four waves' (m, l, O) meet in LDS: [wave][head < g][d + 2]
+  // ---- the waves' (m, l, O) meet in LDS: [wave][head < g][d + 2]
   l += __shfl_xor(l, 16, QIL_WAVE);
   l += __shfl_xor(l, 32, QIL_WAVE);
   const int cell = d + 2;
@@ -172,18 +167,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
         for (int i = 0; i < 4; ++i) mine[t * 16 + 4 * kb + i] = o[t][i];
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < g * d; idx += DEC_THREADS) {
+  for (int idx = threadIdx.x; idx < g * d; idx += blockDim.x) {
     const int h = idx / d, e = idx - h * d;
-    float mw[DEC_WAVES], mm = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) {
-      mw[w] = lds[((size_t)w * g + h) * cell + d];
-      mm = fmaxf(mm, mw[w]);
-    }
+    float mm = -INFINITY;
+    for (int w = 0; w < waves; ++w) mm = fmaxf(mm, lds[((size_t)w * g + h) * cell + d]);
     float total = 0.f, ll = 0.f;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) {
-      const float f = mw[w] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mw[w] - mm) * 1.44269504088896f);
+    for (int w = 0; w < waves; ++w) {                       // fixed order
+      const float mw = lds[((size_t)w * g + h) * cell + d];
+      const float f = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mw - mm) * 1.44269504088896f);
       total += lds[((size_t)w * g + h) * cell + e] * f;
       ll += lds[((size_t)w * g + h) * cell + d + 1] * f;
     }
@@ -200,29 +191,31 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 
 // 1 if the matrix-core decode kernel takes these sizes.
 extern "C" int qil_attn_decode_takes(int heads, int kv_heads, int d, int page_size) {
-  if (heads % kv_heads || d % 16 || d < 16 || d > 256 || page_size % 4) return 0;
+  if (heads % kv_heads || d % 16 || d < 16 || d > 256 || page_size % 8) return 0;
   const int g = heads / kv_heads;
-  return g <= 16 && (size_t)DEC_WAVES * g * (d + 2) * sizeof(float) <= 64 * 1024;
+  return g <= 16 && (size_t)DEC_MAX_WAVES * g * (d + 2) * sizeof(float) <= 64 * 1024;
 }
 
 // Partial results in the layout of the row kernel (acc [rows, heads, parts, d], then m, then l);
-// the caller runs the row kernel's merge when parts > 1.  P must be a multiple of 32.
+// the caller runs the row kernel's merge when parts > 1.  P must be a multiple of 32; a block has
+// `waves` waves (at most 8), best one or two 32-key steps of P for each.
 extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* block_tables, int table_stride, const int* row_seq, const int* positions,
                                const int* row_index, void* workspace, void* out, int rows, int heads, int kv_heads,
-                               int d, int page_size, int window, float scale, int P, int parts, hipStream_t s) {
+                               int d, int page_size, int window, float scale, int P, int parts, int waves,
+                               hipStream_t s) {
   if (rows == 0) return 0;
   if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || P % 32 || P < 32 || parts < 1 || parts > 65535 ||
-      kv_heads > 65535)
+      kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES)
     return -1;
   const int g = heads / kv_heads;
   float* acc = (float*)workspace;
   float* m = acc ? acc + (size_t)rows * heads * parts * d : nullptr;
   float* l = m ? m + (size_t)rows * heads * parts : nullptr;
-  const size_t lds = (size_t)DEC_WAVES * g * (d + 2) * sizeof(float);
+  const size_t lds = (size_t)waves * g * (d + 2) * sizeof(float);
   dim3 grid(rows, kv_heads, parts);
 #define QIL_DEC_CASE(DMAX)                                                                                          \
-  hipLaunchKernelGGL(attn_decode_kernel<DMAX>, grid, dim3(DEC_THREADS), lds, s, (const bf16_t*)q, q_stride,          \
+  hipLaunchKernelGGL(attn_decode_kernel<DMAX>, grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
                      (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
                      row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts)
   if (d <= 64) QIL_DEC_CASE(64);

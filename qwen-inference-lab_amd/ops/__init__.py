@@ -19,8 +19,14 @@ from . import library
 STREAM_GEMM_MAX_ROWS = 16
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
-# Blocks the matrix-core decode kernel aims for (256 CUs; measured best at 8 rows x 2048 keys).
-DECODE_BLOCKS = 512
+# Blocks the matrix-core decode kernel aims for (256 CUs, 8 waves a block; measured best at 8 rows x 2048 keys).
+DECODE_BLOCKS = 256
+# Waves of a block of that kernel; each takes every DECODE_WAVES-th 32-key step of the block's keys.
+DECODE_WAVES = 8
+# Fewest keys of a block of that kernel (more, smaller parts cost more in the merge than they gain).
+DECODE_MIN_PART = 256
+# Most keys of a block.
+DECODE_MAX_PART = 8192
 
 
 class UnsupportedShape(ValueError):
@@ -294,14 +300,14 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         if qkv.dtype == torch.bfloat16 and lib.qil_attn_decode_takes(heads, kv_heads, head_dim, page_size):
             # matrix-core kernel; split the context until the chip has about four blocks per CU
             wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
-            part = min(1024, max(64, -(-(-(-max_context // wanted)) // 64) * 64))
+            part = min(DECODE_MAX_PART, max(DECODE_MIN_PART, -(-(-(-max_context // wanted)) // 64) * 64))
             parts = max(1, -(-max_context // part))
             nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
             workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
             _check(lib.qil_attn_decode(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                        block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                        _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
-                                       window_arg, float(scale), part, parts, _stream()), 'attn_decode')
+                                       window_arg, float(scale), part, parts, DECODE_WAVES, _stream()), 'attn_decode')
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), _ptr(single_rows), _ptr(out), rows, heads,
                                       head_dim, window_arg, part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:
