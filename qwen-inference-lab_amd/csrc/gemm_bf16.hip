@@ -156,7 +156,7 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
 // Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
 #define LINES_WAVES 8
 #define LINES_DEPTH 3                                      // stages of W in flight per wave
-#define LINES_LDS_LIMIT (80 * 1024)                        // two blocks on a CU's 160 KB
+#define LINES_LDS_LIMIT (100 * 1024)                       // one block of 8 waves on a CU when A is long, two otherwise
 
 template <typename OUT>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)

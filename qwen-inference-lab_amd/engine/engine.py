@@ -55,12 +55,14 @@ class Engine:
         try:
             entries = [StepEntry(w.request_id, w.tokens, (len(w.tokens) - 1,) if r else ())
                        for w, r in zip(plan, ready)]
-            logits = self.runner.step(entries)
-            emitted = iter(())
-            if logits is not None:
-                rows = [requests[w.request_id] for w, r in zip(plan, ready) if r]
-                emitted = iter(self.sampler.sample(logits, [SamplingParams(q.temperature, q.seed) for q in rows],
-                                                   [len(q.output) for q in rows]))
+            rows = [requests[w.request_id] for w, r in zip(plan, ready) if r]
+            params, counters = [SamplingParams(q.temperature, q.seed) for q in rows], [len(q.output) for q in rows]
+            fused = getattr(self.runner, 'step_and_sample', None)
+            if fused is not None and isinstance(self.sampler, Sampler):     # the draw rides in the step's launches
+                emitted = iter(fused(entries, self.sampler, params, counters))
+            else:
+                logits = self.runner.step(entries)
+                emitted = iter(self.sampler.sample(logits, params, counters) if logits is not None else ())
         except Exception as error:
             # The failed batch may have written part of its keys and values: retire every member
             # so that none resumes from a partial cache (qil/engine.py:87-93).

@@ -9,12 +9,16 @@ one static int32 device array that is overwritten before each replay; kernels re
 from it and leave early past a row's context, so one graph serves every context up to the
 bucket's end.
 
+With a sampler the draw of the next tokens is part of the graph too (its seeds, output indices and
+temperatures travel in the same array), and a step costs one upload, one replay and one download.
+
 Nothing in the captured region clears memory with a memset node: buffers are allocated, not
 zeroed, and kernels write every element they later read.
 """
 import gc
 import weakref
 
+import numpy as np
 import torch
 
 from .batch import StepEntry
@@ -24,14 +28,20 @@ MAX_GRAPHS = 12
 
 
 class _Graph:
-    def __init__(self, runner, entries, pieces, facts, bucket):
+    def __init__(self, runner, entries, pieces, facts, bucket, sampler=None):
         self.sizes = [len(p) for p in pieces]
-        total = sum(self.sizes)
+        rows = len(entries)
+        self.described = sum(self.sizes)
+        total = self.described + (3 * rows if sampler is not None else 0)
         device = runner.model.device
         self.meta = torch.zeros(total, dtype=torch.int32, device=device)
         self.staging = torch.zeros(total, dtype=torch.int32).pin_memory()
         self.copied = torch.cuda.Event()
-        self.load(pieces)
+        self.drawn = self.drawn_host = None
+        if sampler is not None:
+            self.drawn = torch.zeros((2, rows), dtype=torch.int32, device=device)
+            self.drawn_host = torch.zeros((2, rows), dtype=torch.int32).pin_memory()
+        self.load(pieces, None if sampler is None else np.zeros((3, rows), dtype=np.int32))
         ctx = runner._context(entries, pieces, facts, self.meta, max_context=bucket)
         side = torch.cuda.Stream(device=device)
         side.wait_stream(torch.cuda.current_stream(device))
@@ -46,11 +56,13 @@ class _Graph:
         try:
             with torch.cuda.graph(self.graph):
                 self.logits = runner.model.forward(ctx, runner.views)
+                if sampler is not None:
+                    sampler.draw(self.logits, self.meta[self.described:].view(3, rows), self.drawn)
         finally:
             if collecting:
                 gc.enable()
 
-    def load(self, pieces):
+    def load(self, pieces, packed=None):
         self.copied.synchronize()                           # the previous upload has left the staging buffer
         flat = self.staging.numpy()
         at = 0
@@ -59,6 +71,8 @@ class _Graph:
                 raise RuntimeError('batch layout does not fit the captured graph')
             flat[at:at + size] = piece
             at += size
+        if packed is not None:
+            flat[at:] = packed.reshape(-1)
         self.meta.copy_(self.staging, non_blocking=True)
         self.copied.record()
 
@@ -66,6 +80,14 @@ class _Graph:
         self.load(pieces)
         self.graph.replay()
         return self.logits
+
+    def replay_drawn(self, pieces, packed):
+        """[tokens, finite flags] of the rows, as nested host lists."""
+        self.load(pieces, packed)
+        self.graph.replay()
+        self.drawn_host.copy_(self.drawn, non_blocking=True)
+        torch.cuda.current_stream(self.drawn.device).synchronize()
+        return self.drawn_host.tolist()
 
 
 class DecodeGraphs:
@@ -80,7 +102,9 @@ class DecodeGraphs:
         return self._safe and all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
                    tuple(e[2] if not isinstance(e, StepEntry) else e.want) == (0,) for e in entries) and len(entries) > 0
 
-    def step(self, entries):
+    def step(self, entries, sampler=None, packed=None):
+        """(logits, entries, starts) of a decode batch; with a sampler and its packed parameters the first
+        member is the host copy of the draw ([tokens, finite flags]) instead of logits."""
         runner = self._runner()
         ps = runner.cache.page_size
         normal = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2])) for e in entries]
@@ -92,13 +116,16 @@ class DecodeGraphs:
             bucket = min(bucket, -(-limit // ps) * ps)
         width = -(-bucket // ps)
         entries, pieces, facts = runner._describe(normal, table_width=width, validate=False)
-        key = (len(entries), bucket)
+        key = (len(entries), bucket, sampler is not None)
         graph = self.graphs.get(key)
         if graph is None:
             if len(self.graphs) >= MAX_GRAPHS:
                 self.graphs.pop(next(iter(self.graphs)))
-            graph = self.graphs[key] = _Graph(runner, entries, pieces, facts, bucket)
+            graph = self.graphs[key] = _Graph(runner, entries, pieces, facts, bucket, sampler)
             self.captures += 1
-        logits = graph.replay(pieces).clone()               # the graph's own output buffer is overwritten by the next replay
+        if sampler is not None:
+            result = graph.replay_drawn(pieces, packed)
+        else:
+            result = graph.replay(pieces).clone()           # the graph's own output buffer is overwritten by the next replay
         self.replays += 1
-        return logits, entries, facts['starts']
+        return result, entries, facts['starts']

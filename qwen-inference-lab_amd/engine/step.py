@@ -147,3 +147,27 @@ class ModelRunner:
             self.cache.advance(entry.request, start + len(entry.tokens))
         self.steps += 1
         return logits
+
+    @torch.inference_mode()
+    def step_and_sample(self, entries, sampler, params, counters):
+        """``step``, then ``sampler``'s draw at the wanted places: the tokens as a host list (empty if nothing is
+        wanted).  ``params`` and ``counters`` hold one item per wanted place, in entry order.  For a decode
+        batch the draw is part of the replayed graph."""
+        packed = sampler.pack(params, counters)
+        if self.graphs is not None and self.graphs.takes(entries):
+            drawn, entries, starts = self.graphs.step(entries, sampler, packed)
+        else:
+            entries, ctx = self.prepare(entries)
+            logits = self.model.forward(ctx, self.views)
+            starts = ctx.host_starts
+            drawn = None
+            if logits is not None:
+                if logits.shape[0] != packed.shape[1]:
+                    raise ValueError('one SamplingParams and one counter per wanted place')
+                out = torch.empty((2, logits.shape[0]), dtype=torch.int32, device=logits.device)
+                sampler.draw(logits, torch.from_numpy(packed).to(logits.device), out)
+                drawn = out.tolist()
+        for entry, start in zip(entries, starts):
+            self.cache.advance(entry.request, start + len(entry.tokens))
+        self.steps += 1
+        return sampler.unpack(drawn) if drawn is not None else []

@@ -322,19 +322,21 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
     return out
 
 
-def sample(logits, temperatures, seeds, counters):
+def sample(logits, temperatures, seeds, counters, out=None):
     """float32 [M, V] -> (int32 tokens [M], int32 finite flags [M]).
 
     temperature 0: greedy, lowest index on ties; > 0: seeded Gumbel-max draw from softmax(logits / T)
-    keyed by (seed, counter)."""
+    keyed by (seed, counter).  ``out``: an int32 [2, M] tensor to hold tokens and flags (its rows are returned)."""
     m, vocab = logits.shape
     _require(logits, 'logits', torch.float32)
     _require(temperatures, 'temperatures', torch.float32, (m,))
     _require(seeds, 'seeds', torch.int32, (m,))
     _require(counters, 'counters', torch.int32, (m,))
     lib = library.load()
-    tokens = torch.empty(m, dtype=torch.int32, device=logits.device)
-    finite = torch.empty(m, dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty((2, m), dtype=torch.int32, device=logits.device)
+    _require(out, 'out', torch.int32, (2, m))
+    tokens, finite = out[0], out[1]
     workspace = torch.empty(lib.qil_sample_workspace(m, vocab) // 4, dtype=torch.int32, device=logits.device)
     _check(lib.qil_sample(_ptr(logits), _ptr(temperatures), _ptr(seeds), _ptr(counters), _ptr(tokens), _ptr(finite),
                           _ptr(workspace), m, vocab, _stream()), 'sample')

@@ -8,6 +8,7 @@ depends neither on the batch nor on how the work was cut.
 """
 from dataclasses import dataclass
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -32,16 +33,36 @@ def _int32(value):
 
 
 class Sampler:
+    """``sample`` is the whole thing for logits in hand.  A step function that wants the draw inside its
+    own launch sequence (a captured graph, say) uses the three pieces: ``pack`` on the host, ``draw`` on
+    the device, ``unpack`` on the host."""
+
+    def pack(self, params, counters):
+        """int32 [3, M] host array: seeds, output indices, temperatures (their float32 bits)."""
+        if len(params) != len(counters):
+            raise ValueError('one SamplingParams and one counter per row of logits')
+        packed = np.empty((3, len(params)), dtype=np.int32)
+        packed[0] = [_int32(p.seed) for p in params]
+        packed[1] = [_int32(c) for c in counters]
+        packed[2] = np.asarray([p.temperature for p in params], dtype=np.float32).view(np.int32)
+        return packed
+
+    def draw(self, logits, packed, out):
+        """Device only: ``packed`` int32 [3, M] as ``pack`` makes it, ``out`` int32 [2, M] (tokens, finite flags)."""
+        ops.sample(logits, packed[2].view(torch.float32), packed[0], packed[1], out=out)
+
+    def unpack(self, out):
+        """Tokens from the host copy of ``out`` ([2, M] nested lists); refuses rows with non-finite logits."""
+        tokens, finite = out
+        if not all(finite):
+            raise RuntimeError('model returned non-finite logits')
+        return tokens
+
     def sample(self, logits, params, counters):
         """logits float32 [M, V] on the GPU; params: SamplingParams per row; counters: output index per row."""
-        rows = logits.shape[0]
-        if rows != len(params) or rows != len(counters):
+        if logits.shape[0] != len(params):
             raise ValueError('one SamplingParams and one counter per row of logits')
-        host = torch.tensor([[_int32(p.seed) for p in params], [_int32(c) for c in counters]], dtype=torch.int32)
-        meta = host.to(logits.device)
-        temperatures = torch.tensor([float(p.temperature) for p in params], dtype=torch.float32).to(logits.device)
-        tokens, finite = ops.sample(logits, temperatures, meta[0].contiguous(), meta[1].contiguous())
-        result = torch.stack((tokens, finite)).tolist()
-        if not all(result[1]):
-            raise RuntimeError('model returned non-finite logits')
-        return result[0]
+        packed = torch.from_numpy(self.pack(params, counters)).to(logits.device)
+        out = torch.empty((2, logits.shape[0]), dtype=torch.int32, device=logits.device)
+        self.draw(logits, packed, out)
+        return self.unpack(out.tolist())

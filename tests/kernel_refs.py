@@ -131,10 +131,14 @@ def sample_scores(logits, temperatures, seeds, counters):
     return torch.stack(rows)
 
 
-def sample(logits, temperatures, seeds, counters):
+def sample(logits, temperatures, seeds, counters, out=None):
     scores = sample_scores(logits, temperatures, seeds, counters)
     finite = torch.isfinite(logits).all(dim=-1).to(torch.int32)
-    return scores.argmax(dim=-1).to(torch.int32), finite
+    tokens = scores.argmax(dim=-1).to(torch.int32)
+    if out is not None:
+        out[0], out[1] = tokens, finite
+        return out[0], out[1]
+    return tokens, finite
 
 
 ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
