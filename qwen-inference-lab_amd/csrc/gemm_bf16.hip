@@ -155,13 +155,66 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
 // LDS operations of one wave complete in program order, so the buffer needs no barrier.
 // Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
 #define LINES_WAVES 8
+
+// A given as the unmerged partial results of split-context attention (attention_rows.hip,
+// attention_decode.hip): acc [M, heads, parts, d], m and l [M, heads, parts], float32.  Row m, column
+// head * d + e of A is sum_p acc_p[e] exp(m_p - max m) / sum_p l_p exp(m_p - max m) over the parts that
+// hold keys of the row: the merge of attn_rows_merge_kernel, made while A is staged.
+struct UnmergedA {
+  const float* acc;
+  const float* m;
+  const float* l;
+  const int* positions;                                    // [M]: a row's context is its position + 1
+  int heads, d, parts, P, window;
+};
 #define LINES_DEPTH 3                                      // stages of W in flight per wave
 #define LINES_LDS_LIMIT (100 * 1024)                       // one block of 8 waves on a CU when A is long, two otherwise
 
-template <typename OUT>
+// Eight merged values of row m starting at column k (all of one head: d % 8 == 0), as bfloat16.
+__device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
+  const int head = k / u.d, e = k - head * u.d;
+  const int ctx = u.positions[m] + 1;
+  const int lo = u.window > 0 ? max(0, ctx - u.window) : 0;
+  const int first = lo / u.P, last = (ctx - 1) / u.P;
+  const size_t cell0 = ((size_t)m * u.heads + head) * u.parts;
+  // four parts at a time, all their loads first: a loop that waits for memory once per part would
+  // cost more than the merge kernel it replaces
+  float top = -INFINITY;
+  for (int p0 = first; p0 <= last; p0 += 4) {
+    float mv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mv[j] = u.m[cell0 + min(p0 + j, last)];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) top = fmaxf(top, mv[j]);
+  }
+  float denom = 0.f, numer[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int p0 = first; p0 <= last; p0 += 4) {
+    float mv[4], lv[4], part[4][8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int p = min(p0 + j, last);
+      mv[j] = u.m[cell0 + p];
+      lv[j] = u.l[cell0 + p];
+      ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                           // the order and the arithmetic of the merge kernel
+      if (p0 + j <= last) {
+        const float f = expf(mv[j] - top);
+        denom += lv[j] * f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) numer[i] += part[j][i] * f;
+      }
+    }
+  }
+  return make_uint4(pack_bf16(numer[0] / denom, numer[1] / denom), pack_bf16(numer[2] / denom, numer[3] / denom),
+                    pack_bf16(numer[4] / denom, numer[5] / denom), pack_bf16(numer[6] / denom, numer[7] / denom));
+}
+
+template <typename OUT, bool MERGE>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
-gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N,
-                       int K, int cols_per_split) {
+gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const bf16_t* __restrict__ W,
+                       OUT* __restrict__ C, int M, int N, int K, int cols_per_split) {
   extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
@@ -185,7 +238,7 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
   for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
     const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
     uint4 v = make_uint4(0, 0, 0, 0);
-    if (m < M) v = *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
+    if (m < M) v = MERGE ? merged8(unmerged, m, k_begin + c) : *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
     *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
   }
   // Every wave walks its K range from a start of its own and wraps around: waves that all read the
@@ -257,10 +310,11 @@ static bool lines_takes(const void* A, const void* W, const float* bias, int M, 
   return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
 }
 
-template <typename OUT>
-static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
+template <typename OUT, bool MERGE = false>
+static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
+                        UnmergedA unmerged = UnmergedA()) {
   const size_t lds = lines_lds(M, K, splits);
-  auto kernel = gemm_bf16_lines_kernel<OUT>;
+  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE>;
   static size_t granted = 0;                              // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -268,7 +322,7 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
     granted = lds;
   }
   dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
-  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, unmerged, W, C, M, N, K, K / splits);
   return 0;
 }
 
@@ -495,6 +549,34 @@ extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
   int code, splits;
   plan(M, N, K, true, &code, &splits);
   return splits;
+}
+
+// 1 if qil_gemm_bf16_unmerged takes these sizes (rows, output columns, heads, head size, K splits).
+extern "C" int qil_gemm_bf16_unmerged_takes(int M, int N, int heads, int d, int splits) {
+  const long K = (long)heads * d;
+  if (M < 1 || M > 16 || N < 1 || d % 8 || splits < 1 || K > (1 << 30) || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH)
+    return 0;
+  return lines_lds(M, (int)K, splits) <= LINES_LDS_LIMIT;
+}
+
+// C float32 [splits, M, N] = partial sums of merge(workspace) W^T, the merge being that of qil_attn_merge
+// over a workspace laid out as qil_attn_rows_workspace describes (rows 0 .. M-1, no row index), made
+// while the whole-line kernel stages A; K = heads * d.
+extern "C" int qil_gemm_bf16_unmerged(const void* workspace, const int* positions, const void* W, void* C, int M, int N,
+                                      int heads, int d, int window, int P, int parts, int splits, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  if (!qil_gemm_bf16_unmerged_takes(M, N, heads, d, splits) || parts < 1 || P < 1 || ((uintptr_t)W % 16) ||
+      ((uintptr_t)workspace % 16))
+    return -1;
+  UnmergedA u;
+  u.acc = (const float*)workspace;
+  u.m = u.acc + (size_t)M * heads * parts * d;
+  u.l = u.m + (size_t)M * heads * parts;
+  u.positions = positions;
+  u.heads = heads; u.d = d; u.parts = parts; u.P = P; u.window = window;
+  const int status = launch_lines<float, true>(nullptr, (const bf16_t*)W, (float*)C, M, N, heads * d, splits, s, u);
+  if (status) return status;
+  QIL_RETURN_LAUNCH_STATUS();
 }
 
 // out_dtype QIL_BF16: C bfloat16 [M, N], splits must be 1.  QIL_F32: C float32 [splits, M, N], the

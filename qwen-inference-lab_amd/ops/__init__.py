@@ -45,6 +45,23 @@ class Partials:
         return self.tensor.sum(dim=0)
 
 
+class Unmerged:
+    """Attention of single rows left as the float32 partial results of the context's parts (rows 0 .. N-1
+    of the step, all alone in their sequences).  ``merge()`` gives the [N, heads * d] tensor; ``linear``
+    takes it as it is and merges while it stages its operand."""
+
+    def __init__(self, workspace, positions, out, *, heads, head_dim, window, part, parts):
+        self.workspace, self.positions, self.out = workspace, positions, out
+        self.heads, self.head_dim, self.window, self.part, self.parts = heads, head_dim, window, part, parts
+        self.shape, self.dtype, self.device = tuple(out.shape), out.dtype, out.device
+
+    def merge(self):
+        _check(library.load().qil_attn_merge(_ptr(self.workspace), _ptr(self.positions), None, _ptr(self.out),
+                                             self.shape[0], self.heads, self.head_dim, self.window, self.part,
+                                             self.parts, _code(self.dtype), _stream()), 'attn_merge')
+        return self.out
+
+
 def _operand(value, name, model_dtype, shape):
     """(pointer, dtype code, splits) of a consumer's input: a tensor of the model's type or Partials."""
     if isinstance(value, Partials):
@@ -152,7 +169,22 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     """x [N, K] @ weight [O, K]^T (+ bias float32 [O]) -> [N, O] in out_dtype (default: x's).
 
     ``partials=True`` allows the result to come back as ``Partials`` (bfloat16 products with few
-    rows: float32, K split over blocks) for a consumer that adds them; otherwise a tensor."""
+    rows: float32, K split over blocks) for a consumer that adds them; otherwise a tensor.
+    ``x`` may be ``Unmerged`` attention results."""
+    if isinstance(x, Unmerged):
+        lib = library.load()
+        n, k = x.shape
+        o = weight.shape[0]
+        _require(weight, 'weight', x.dtype, (o, k))
+        splits = lib.qil_gemm_bf16_splits(n, o, k)
+        if partials and bias is None and out_dtype in (None, x.dtype) and x.dtype == torch.bfloat16 and \
+                lib.qil_gemm_bf16_unmerged_takes(n, o, x.heads, x.head_dim, splits):
+            out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+            _check(lib.qil_gemm_bf16_unmerged(_ptr(x.workspace), _ptr(x.positions), _ptr(weight), _ptr(out), n, o,
+                                              x.heads, x.head_dim, x.window, x.part, x.parts, splits, _stream()),
+                   'gemm_bf16_unmerged')
+            return Partials(out)
+        x = x.merge()
     _require(x, 'x')
     _require(weight, 'weight', x.dtype)
     n, k = x.shape
@@ -258,7 +290,8 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
-                    cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window):
+                    cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
+                    unmerged=False):
     """Attention of every row of the step over its request's cached keys.
 
     ``q`` [N, heads * head_dim] (head h at columns [h d, (h + 1) d)).  Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
@@ -266,7 +299,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
 
     Sequences with two or more rows (``cu_seqlens``, ``seq_starts``) go to the matrix-core tile
     kernel; rows alone in their sequence (``single_rows``: their indices, or None when every row is
-    alone, i.e. ``max_query == 1``) go to the split-context row kernel.
+    alone, i.e. ``max_query == 1``) go to the split-context row kernel.  With ``unmerged`` the result may
+    come back as ``Unmerged`` (every row alone, context in several parts) for ``linear`` to merge.
     """
     n = q.shape[0]
     qkv = q
@@ -308,6 +342,9 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                                        block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                        _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
                                        window_arg, float(scale), part, parts, DECODE_WAVES, _stream()), 'attn_decode')
+            if unmerged and parts > 1 and single_rows is None:
+                return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
+                                part=part, parts=parts)
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), _ptr(single_rows), _ptr(out), rows, heads,
                                       head_dim, window_arg, part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:

@@ -156,6 +156,9 @@ def _declare(lib):
     lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_gemm_bf16_splits.argtypes = [i, i, i]
     lib.qil_gemm_bf16_splits.restype = i
+    lib.qil_gemm_bf16_unmerged.argtypes = [p, p, p, p, i, i, i, i, i, i, i, i, p]
+    lib.qil_gemm_bf16_unmerged_takes.argtypes = [i, i, i, i, i]
+    lib.qil_gemm_bf16_unmerged_takes.restype = i
     lib.qil_gemm_bf16_gated.argtypes = [p, p, p, i, i, i, i, i, i, p]
     lib.qil_gemm_bf16_gated_takes.argtypes = [i, i, i]
     lib.qil_gemm_bf16_gated_takes.restype = i
@@ -163,5 +166,5 @@ def _declare(lib):
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z
     for name in ('qil_embed', 'qil_add_rmsnorm', 'qil_silu_mul', 'qil_add_bias', 'qil_qk_norm_rope_store',
-                 'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_gemm_bf16_gated', 'qil_sample'):
+                 'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_gemm_bf16_gated', 'qil_gemm_bf16_unmerged', 'qil_sample'):
         getattr(lib, name).restype = i

@@ -69,5 +69,5 @@ class Attention(Mixer):
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
             max_query=ctx.max_query, max_context=ctx.max_context,
-            scale=self.scale, window=self.window)
+            scale=self.scale, window=self.window, unmerged=True)
         return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

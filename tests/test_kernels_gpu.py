@@ -319,6 +319,38 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
         torch.testing.assert_close(ops.paged_attention(qkv, **args)[0], got[0], atol=0, rtol=0)
 
 
+@pytest.mark.parametrize('lengths,window,d,heads,kv_heads,out_features', [
+    ([2100, 1, 700, 1290, 64, 2047, 300, 1500], None, 128, 32, 8, 4096),
+    ([900, 2100, 33], 500, 128, 32, 4, 300),
+    ([5000], None, 128, 32, 8, 1024),
+    ([600, 700], None, 64, 8, 2, 300),                      # too short a K for the fused path: merged first
+])
+def test_linear_merges_unmerged_attention(ops, lengths, window, d, heads, kv_heads, out_features):
+    """The output projection takes attention results whose context parts are not merged yet and merges
+    them while it stages its operand: bit for bit what the merge kernel followed by the product gives."""
+    dtype, page_size = torch.bfloat16, 16
+    k_cache, v_cache, table, _ = build_cache(lengths, page_size, kv_heads, d, dtype)
+    rows = len(lengths)
+    q = rand(rows, heads * d, dtype=dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
+                block_tables=table, row_seq=torch.arange(rows, dtype=torch.int32).cuda(), positions=positions,
+                cu_seqlens=None, seq_starts=None, single_rows=None, n_seqs=rows, max_query=1, max_context=max(lengths),
+                scale=d ** -0.5, window=window)
+    w = rand(out_features, heads * d, dtype=dtype, seed=3, scale=(heads * d) ** -0.5)
+    merged = ops.paged_attention(q, **args)
+    assert isinstance(merged, torch.Tensor)
+    want = ops.linear(merged, w, None, partials=True)
+    lazy = ops.paged_attention(q, unmerged=True, **args)
+    assert isinstance(lazy, ops.Unmerged), 'several context parts and only single rows: nothing to merge yet'
+    got = ops.linear(lazy, w, None, partials=True)
+    assert isinstance(got, ops.Partials) and isinstance(want, ops.Partials)
+    torch.testing.assert_close(got.tensor, want.tensor, atol=0, rtol=0)
+    torch.testing.assert_close(lazy.merge(), merged, atol=0, rtol=0)
+    biased = ops.linear(ops.paged_attention(q, unmerged=True, **args), w, rand(out_features, seed=5))     # no fused path: merges first
+    check(biased, merged.double() @ w.double().t() + rand(out_features, seed=5).double(), dtype, scale=2)
+
+
 def mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, window, scale=0.3):
     """Sequences of `lengths` cached tokens whose last `chunks[i]` positions are this step's rows."""
     k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
