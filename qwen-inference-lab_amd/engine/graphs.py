@@ -37,6 +37,9 @@ class _Graph:
         self.meta = torch.zeros(total, dtype=torch.int32, device=device)
         self.staging = torch.zeros(total, dtype=torch.int32).pin_memory()
         self.copied = torch.cuda.Event()
+        self.offsets = np.cumsum([0] + self.sizes).tolist()
+        self.widths = list(facts['widths'])
+        self.written = [[(None, 0)] * rows for _ in self.widths]     # per page group and row: (table, entries uploaded)
         self.drawn = self.drawn_host = None
         if sampler is not None:
             self.drawn = torch.zeros((2, rows), dtype=torch.int32, device=device)
@@ -76,14 +79,52 @@ class _Graph:
         self.meta.copy_(self.staging, non_blocking=True)
         self.copied.record()
 
-    def replay(self, pieces):
-        self.load(pieces)
+    def refresh(self, runner, entries, packed=None):
+        """``load`` for the steps after the first, straight from the requests' state: only what changes from
+        one decode step to the next is rewritten (tokens, positions, slots, and the block tables' new
+        entries; a table is a list that only grows, apart from given-back entries that no kernel reads).
+        Holds the pages of the new tokens.  Returns the requests' positions."""
+        cache = runner.cache
+        ps, offsets = cache.page_size, self.offsets
+        starts = [cache.computed[e.request] for e in entries]
+        for entry, start in zip(entries, starts):
+            cache.ensure(entry.request, start + 1)
+        self.copied.synchronize()
+        flat = self.staging.numpy()
+        flat[offsets[0]:offsets[1]] = [e.tokens[0] for e in entries]
+        flat[offsets[1]:offsets[2]] = starts                # positions
+        flat[offsets[4]:offsets[5]] = starts                # where the requests' rows begin
+        flat[offsets[5]:offsets[6]] = [cache.slots[e.request] for e in entries]
+        for group, width in enumerate(self.widths):
+            tables_at, slots_at, written = offsets[8 + 2 * group], offsets[9 + 2 * group], self.written[group]
+            for row, (entry, start) in enumerate(zip(entries, starts)):
+                table = cache.table(group, entry.request)
+                count = len(table)
+                if count > width:
+                    raise RuntimeError('batch layout does not fit the captured graph')
+                known, done = written[row]
+                if known is not table or done > count:
+                    done = 0
+                if done < count:
+                    at = tables_at + row * width
+                    flat[at + done:at + count] = [max(page, 0) for page in table[done:]]
+                    written[row] = (table, count)
+                page = table[start // ps]
+                if page < 0:
+                    raise RuntimeError('a new token falls into a page that was given back')
+                flat[slots_at + row] = page * ps + start % ps
+        if packed is not None:
+            flat[self.described:] = packed.reshape(-1)
+        self.meta.copy_(self.staging, non_blocking=True)
+        self.copied.record()
+        return starts
+
+    def run(self):
         self.graph.replay()
         return self.logits
 
-    def replay_drawn(self, pieces, packed):
+    def run_drawn(self):
         """[tokens, finite flags] of the rows, as nested host lists."""
-        self.load(pieces, packed)
         self.graph.replay()
         self.drawn_host.copy_(self.drawn, non_blocking=True)
         torch.cuda.current_stream(self.drawn.device).synchronize()
@@ -115,17 +156,18 @@ class DecodeGraphs:
         if limit is not None:
             bucket = min(bucket, -(-limit // ps) * ps)
         width = -(-bucket // ps)
-        entries, pieces, facts = runner._describe(normal, table_width=width, validate=False)
-        key = (len(entries), bucket, sampler is not None)
+        key = (len(normal), bucket, sampler is not None)
         graph = self.graphs.get(key)
         if graph is None:
             if len(self.graphs) >= MAX_GRAPHS:
                 self.graphs.pop(next(iter(self.graphs)))
-            graph = self.graphs[key] = _Graph(runner, entries, pieces, facts, bucket, sampler)
+            described, pieces, facts = runner._describe(normal, table_width=width, validate=False)
+            graph = self.graphs[key] = _Graph(runner, described, pieces, facts, bucket, sampler)
             self.captures += 1
+        starts = graph.refresh(runner, normal, packed)
         if sampler is not None:
-            result = graph.replay_drawn(pieces, packed)
+            result = graph.run_drawn()
         else:
-            result = graph.replay(pieces).clone()           # the graph's own output buffer is overwritten by the next replay
+            result = graph.run().clone()                    # the graph's own output buffer is overwritten by the next replay
         self.replays += 1
-        return result, entries, facts['starts']
+        return result, normal, starts
