@@ -453,6 +453,13 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
   return (int)hipGetLastError();
 }
 
+// The branch-free kernel for the common bfloat16 case (attention_tile_bf16.hip).
+extern "C" int qil_attn_tile_bf16_takes(int d, int page_size, int table_stride);
+extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                  const int* block_tables, int table_stride, const int* cu_seqlens,
+                                  const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                  int d, int page_size, int window, float scale, hipStream_t s);
+
 // Sequences with >= 2 rows.  q: rows of stride q_stride, head h at h * d; out [rows, heads * d].
 // Requires d % 8 == 0, 8 <= d <= 256.  Returns -1 on a size it does not take.
 extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache,
@@ -461,6 +468,9 @@ extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, c
                              int window, float scale, int dtype, hipStream_t s) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
+  if (dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
+    return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);
 #define QIL_TILE_CASE(T, DMAX)                                                                                      \
   return launch_tile<T, DMAX, (sizeof(T) == 2 && DMAX <= 128) ? 2 : 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s)

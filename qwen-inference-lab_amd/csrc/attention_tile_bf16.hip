@@ -1,0 +1,321 @@
+// The tile kernel of attention_tile.hip for its common case, written without branches in the tile loop:
+// bfloat16, head size exactly D (64, 128 or 256), page_size % 8 == 0, a block table of a sequence that
+// fits in LDS.  Same block shape, same matrix-core formulation, same order of every sum, so a row gets
+// bit for bit the result of the general kernel (qil/model.py:59-66 is the formula of both).
+//
+// What differs is the schedule:
+//  * the sequence's block-table entries are copied to LDS once, so finding a page is an LDS read and
+//    not a load that the K and V loads must wait for;
+//  * while a tile is multiplied, the next tile's K and V^T vectors are already on their way into
+//    registers (they are written to LDS after the barrier that ends the tile);
+//  * a tile is multiplied by one of two straight-line bodies: one for tiles of which every key is
+//    visible to every row of the wave, one that masks (the diagonal, the window's edge, the rows past
+//    the sequence's end).  No size is tested inside them, so the compiler can start the LDS reads of a
+//    fragment while the products of the one before run.
+#include <type_traits>
+
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define FAST_THREADS 256
+#define FAST_BK 64                                         // keys per LDS tile
+#define FAST_PAD 8                                         // LDS row padding in elements
+#define FAST_TABLE_MAX 4096                                // block-table entries of a sequence kept in LDS
+
+template <int D, int RB>
+__global__ void __launch_bounds__(FAST_THREADS, 2)
+attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                      const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
+                      const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
+                      int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift) {
+  constexpr int BK = FAST_BK, QFRAGS = D / 32, DTILES = D / 16, SUB = BK / 16;
+  constexpr int K_ROW = D + FAST_PAD, V_ROW = BK + FAST_PAD;
+  constexpr int K_ITERS = BK * (D / 8) / FAST_THREADS, V_ITERS = D * (BK / 8) / FAST_THREADS;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);         // [BK][K_ROW]
+  bf16_t* Vt = Ks + BK * K_ROW;                            // [D][V_ROW]
+  int* pages = reinterpret_cast<int*>(Vt + D * V_ROW);     // the block-table entries this block needs
+
+  const int seq = blockIdx.y;
+  const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
+  if (n < 2) return;
+  const int RT = 4 / GH;
+  const int block_rows = 16 * RB * RT;
+  // consecutive groups of 256 blocks walk the row tiles in opposite directions (as the general kernel does)
+  const int linear = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int across = ((linear >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int tile_row0 = across * block_rows;
+  if (tile_row0 >= n) return;
+  const int kvh = blockIdx.z / chunks, chunk = blockIdx.z % chunks;
+  const int g = heads / kv_heads;
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int head_local = chunk * GH + wave % GH, row_group = wave / GH;
+  const int wave_row0 = tile_row0 + row_group * 16 * RB;
+  const bool wave_active = head_local < g && wave_row0 < n;
+  const int head = kvh * g + head_local;
+  const int start = seq_starts[seq];
+
+  const int rows_in_block = min(block_rows, n - tile_row0);
+  const int pos_first = start + tile_row0;
+  const int key_end = pos_first + rows_in_block;                       // last position + 1
+  const int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  const int first_tile = key_begin / BK * BK;
+
+  // block-table entries of [first_tile, key_end) into LDS
+  const int first_page = ps_shift >= 0 ? first_tile >> ps_shift : first_tile / page_size;
+  const int last_page = ps_shift >= 0 ? (key_end - 1) >> ps_shift : (key_end - 1) / page_size;
+  {
+    const int* table = block_tables + (size_t)seq * table_stride;
+    for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS) pages[i] = table[first_page + i];
+  }
+
+  int my_row[RB], my_pos[RB];
+  bool row_valid[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    my_row[b] = wave_row0 + b * 16 + r;
+    row_valid[b] = wave_active && my_row[b] < n;
+    my_pos[b] = row_valid[b] ? start + my_row[b] : -1;     // a row past the end sees no key
+  }
+  const int wave_last_pos = start + min(n, wave_row0 + 16 * RB) - 1;   // nothing beyond it is visible to this wave
+
+  // Q fragments: B operands, Q[row r of tile b][dims 32 ks + 8 kb ..]
+  bf16x8 qb[RB][QFRAGS];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const bf16_t* qrow = q + (size_t)(q0 + (row_valid[b] ? my_row[b] : 0)) * q_stride + (size_t)(wave_active ? head : 0) * D;
+#pragma unroll
+    for (int ks = 0; ks < QFRAGS; ++ks) {
+      uint4 raw = make_uint4(0, 0, 0, 0);
+      if (row_valid[b]) raw = *reinterpret_cast<const uint4*>(qrow + ks * 32 + kb * 8);
+      qb[b][ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+  float m[RB], l[RB];
+  f32x4 o[RB][DTILES];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    m[b] = -INFINITY;
+    l[b] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DTILES; ++t) o[b][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // What this thread stages of every tile: K vector it = 16 bytes of key idx / (D / 8), V^T vector it =
+  // 8 keys (one 16-byte piece of a page row) of dim idx % D.
+  // Addresses: 64 bits for the page (a cache may hold more than 2^31 elements), 32 bits within it.
+  uint4 k_reg[K_ITERS], v_reg[V_ITERS];
+  const size_t page_stride = (size_t)kv_heads * page_size * D;
+  const uint32_t k_head = (uint32_t)kvh * page_size * D, v_head = (uint32_t)kvh * D * page_size;
+  auto request = [&](int k0) {
+#pragma unroll
+    for (int it = 0; it < K_ITERS; ++it) {
+      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
+      const int key = min(max(k0 + kl, key_begin), key_end - 1);     // clamped onto a needed key; zeroed when published
+      const int block = ps_shift >= 0 ? key >> ps_shift : key / page_size;
+      const uint32_t offset = key - block * page_size;
+      k_reg[it] = *reinterpret_cast<const uint4*>(k_cache + (size_t)pages[block - first_page] * page_stride +
+                                                  (k_head + offset * D + dv));
+    }
+#pragma unroll
+    for (int it = 0; it < V_ITERS; ++it) {
+      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int grp = idx / D, dim = idx % D;
+      const int key = min(max(k0 + grp * 8, key_begin & ~7), (key_end - 1) & ~7);
+      const int block = ps_shift >= 0 ? key >> ps_shift : key / page_size;
+      const uint32_t offset = key - block * page_size;
+      v_reg[it] = *reinterpret_cast<const uint4*>(v_cache + (size_t)pages[block - first_page] * page_stride +
+                                                  (v_head + (uint32_t)dim * page_size + offset));
+    }
+  };
+  auto publish = [&](int k0) {
+    const bool inside = k0 >= key_begin && k0 + BK <= key_end;        // no key of the tile needs zeroing
+#pragma unroll
+    for (int it = 0; it < K_ITERS; ++it) {
+      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
+      const int key = k0 + kl;
+      const bool valid = inside || (key >= key_begin && key < key_end);
+      *reinterpret_cast<uint4*>(Ks + kl * K_ROW + dv) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < V_ITERS; ++it) {
+      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int grp = idx / D, dim = idx % D;
+      uint4 raw = v_reg[it];
+      if (!inside) {       // zero what lies outside [key_begin, key_end): never written, or someone else's
+        const int key = k0 + grp * 8;
+        uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (!(key + e >= key_begin && key + e < key_end)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+        raw = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+      *reinterpret_cast<uint4*>(Vt + dim * V_ROW + grp * 8) = raw;
+    }
+  };
+
+  // One tile's arithmetic.  MASKED: keys a row does not see get score -inf (probability 0).
+  const float c = scale * 1.44269504088896f;               // p = exp2((s - m) c): the scale enters in the exponent
+  auto attend = [&](int k0, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    f32x4 s[RB][SUB];
+#pragma unroll
+    for (int jt = 0; jt < SUB; ++jt) {
+      const bf16_t* krow = Ks + (jt * 16 + r) * K_ROW + kb * 8;
+#pragma unroll
+      for (int b = 0; b < RB; ++b) s[b][jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < QFRAGS; ++ks) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + ks * 32));
+#pragma unroll
+        for (int b = 0; b < RB; ++b) s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[b][ks], s[b][jt], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int jt = 0; jt < SUB; ++jt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (MASKED) {
+            const int key = k0 + jt * 16 + 4 * kb + i;
+            const bool visible = key <= my_pos[b] && (window <= 0 || key > my_pos[b] - window);
+            s[b][jt][i] = visible ? s[b][jt][i] : -INFINITY;
+          }
+          mx = fmaxf(mx, s[b][jt][i]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+      const float m_new = fmaxf(m[b], mx);
+      const float base = (m_new == -INFINITY) ? 0.f : m_new;                              // exp(-inf - 0) = 0
+      const float shift = -base * c;
+      const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(fmaf(m[b], c, shift));
+      float psum = 0.f;
+#pragma unroll
+      for (int jt = 0; jt < SUB; ++jt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[b][jt][i], c, shift));
+          s[b][jt][i] = p;
+          psum += p;
+        }
+      l[b] = l[b] * alpha + psum;
+      if (m_new != m[b]) {                       // nothing to rescale while the maximum stands
+#pragma unroll
+        for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[b][t][i] *= alpha;
+      }
+      m[b] = m_new;
+    }
+#pragma unroll
+    for (int st = 0; st < SUB / 2; ++st) {
+      bf16x8 pb[RB];
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        uint32_t packed[4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          packed[i] = pack_bf16(s[b][2 * st][2 * i], s[b][2 * st][2 * i + 1]);
+          packed[2 + i] = pack_bf16(s[b][2 * st + 1][2 * i], s[b][2 * st + 1][2 * i + 1]);
+        }
+        pb[b] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+      }
+#pragma unroll
+      for (int t = 0; t < DTILES; ++t) {
+        const bf16_t* vrow = Vt + (t * 16 + r) * V_ROW + st * 32 + 4 * kb;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+#pragma unroll
+        for (int b = 0; b < RB; ++b) o[b][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[b], o[b][t], 0, 0, 0);
+      }
+    }
+  };
+
+  __syncthreads();                                         // the table entries are in place
+  request(first_tile);
+  for (int k0 = first_tile; k0 < key_end; k0 += BK) {
+    __syncthreads();                                       // the previous tile is consumed
+    publish(k0);
+    __syncthreads();
+    if (k0 + BK < key_end) request(k0 + BK);
+    if (wave_active && k0 <= wave_last_pos) {
+      const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 16 * RB <= n &&
+                               (window <= 0 || k0 > wave_last_pos - window);
+      if (all_visible) attend(k0, std::false_type());
+      else attend(k0, std::true_type());
+    }
+  }
+
+  if (!wave_active) return;
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    float total = l[b];
+    total += __shfl_xor(total, 16, QIL_WAVE);
+    total += __shfl_xor(total, 32, QIL_WAVE);
+    if (!row_valid[b]) continue;
+    const float inv = 1.f / total;
+    bf16_t* orow = out + ((size_t)(q0 + my_row[b]) * heads + head) * D;
+#pragma unroll
+    for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st(orow + t * 16 + 4 * kb + i, o[b][t][i] * inv);
+  }
+}
+
+template <int D, int RB>
+static int launch_fast(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                       int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
+                       int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s) {
+  const int g = heads / kv_heads;
+  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
+  const size_t lds = ((size_t)FAST_BK * (D + FAST_PAD) + (size_t)D * (FAST_BK + FAST_PAD)) * sizeof(bf16_t) +
+                     (size_t)table_stride * sizeof(int);
+  auto kernel = attn_tile_bf16_kernel<D, RB>;
+  static size_t granted = 0;                     // per instantiation
+  if (lds > 64 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks);
+  int ps_shift = -1;                                      // log2 of a power-of-two page size
+  for (int b = 0; b < 30; ++b)
+    if (page_size == (1 << b)) ps_shift = b;
+  hipLaunchKernelGGL(kernel, grid, dim3(FAST_THREADS), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+                     (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
+                     kv_heads, page_size, window, scale, GH, chunks, ps_shift);
+  return (int)hipGetLastError();
+}
+
+// 1 if the kernel of this file takes the sizes (bfloat16 only).
+extern "C" int qil_attn_tile_bf16_takes(int d, int page_size, int table_stride) {
+  return (d == 64 || d == 128 || d == 256) && page_size > 0 && page_size % 8 == 0 && table_stride >= 1 &&
+         table_stride <= FAST_TABLE_MAX;
+}
+
+// The arguments of qil_attn_tile (attention_tile.hip), which calls this when the sizes are taken.
+extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                  const int* block_tables, int table_stride, const int* cu_seqlens,
+                                  const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                  int d, int page_size, int window, float scale, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if (!qil_attn_tile_bf16_takes(d, page_size, table_stride) || heads % kv_heads || n_seqs > 65535 ||
+      kv_heads * 2 > 65535)
+    return -1;
+  if (d == 64)
+    return launch_fast<64, 2>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                              n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+  if (d == 128)
+    return launch_fast<128, 2>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                               n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+  return launch_fast<256, 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                             n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+}
