@@ -11,7 +11,11 @@
 //  * a tile is multiplied by one of two straight-line bodies: one for tiles of which every key is
 //    visible to every row of the wave, one that masks (the diagonal, the window's edge, the rows past
 //    the sequence's end).  No size is tested inside them, so the compiler can start the LDS reads of a
-//    fragment while the products of the one before run.
+//    fragment while the products of the one before run;
+//  * the rows of a 16-key score tile are assigned to keys so that a lane's eight probabilities of a
+//    32-key step belong to eight consecutive keys: its V^T fragment is one 16-byte LDS read;
+//  * for D <= 128 the LDS holds two tiles, so a tile costs one barrier: the next tile is written to
+//    the other half before this one is multiplied.
 #include <type_traits>
 
 #include "common.h"
@@ -34,9 +38,10 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   constexpr int K_ROW = D + FAST_PAD, V_ROW = BK + FAST_PAD;
   constexpr int K_ITERS = BK * (D / 8) / FAST_THREADS, V_ITERS = D * (BK / 8) / FAST_THREADS;
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  bf16_t* Ks = reinterpret_cast<bf16_t*>(lds_raw);         // [BK][K_ROW]
-  bf16_t* Vt = Ks + BK * K_ROW;                            // [D][V_ROW]
-  int* pages = reinterpret_cast<int*>(Vt + D * V_ROW);     // the block-table entries this block needs
+  constexpr bool TWO = D <= 128;                           // two tiles in LDS
+  constexpr int TILE_ELEMS = BK * K_ROW + D * V_ROW;       // K [BK][K_ROW] (rows in score-tile order), then V^T [D][V_ROW]
+  bf16_t* tiles = reinterpret_cast<bf16_t*>(lds_raw);
+  int* pages = reinterpret_cast<int*>(tiles + (TWO ? 2 : 1) * TILE_ELEMS);   // the block-table entries this block needs
 
   const int seq = blockIdx.y;
   const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
@@ -132,7 +137,11 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
                                                   (v_head + (uint32_t)dim * page_size + offset));
     }
   };
-  auto publish = [&](int k0) {
+  // Key kl of a tile (= 32 a + 8 b + 4 c + e) is row 4 b + e of score sub-tile 2 a + c: lane (r, kb) of the
+  // score product then holds, in sub-tiles 2 a and 2 a + 1, the keys 32 a + 8 kb .. + 7.
+  auto publish = [&](int k0, bf16_t* tile) {
+    bf16_t* Ks = tile;
+    bf16_t* Vt = tile + BK * K_ROW;
     const bool inside = k0 >= key_begin && k0 + BK <= key_end;        // no key of the tile needs zeroing
 #pragma unroll
     for (int it = 0; it < K_ITERS; ++it) {
@@ -140,7 +149,8 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
       const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
       const int key = k0 + kl;
       const bool valid = inside || (key >= key_begin && key < key_end);
-      *reinterpret_cast<uint4*>(Ks + kl * K_ROW + dv) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
+      const int row = ((kl >> 5) * 2 + ((kl >> 2) & 1)) * 16 + ((kl >> 3) & 3) * 4 + (kl & 3);
+      *reinterpret_cast<uint4*>(Ks + row * K_ROW + dv) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int it = 0; it < V_ITERS; ++it) {
@@ -161,8 +171,10 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
 
   // One tile's arithmetic.  MASKED: keys a row does not see get score -inf (probability 0).
   const float c = scale * 1.44269504088896f;               // p = exp2((s - m) c): the scale enters in the exponent
-  auto attend = [&](int k0, auto masked_tag) {
+  auto attend = [&](int k0, const bf16_t* tile, auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
+    const bf16_t* Ks = tile;
+    const bf16_t* Vt = tile + BK * K_ROW;
     f32x4 s[RB][SUB];
 #pragma unroll
     for (int jt = 0; jt < SUB; ++jt) {
@@ -184,7 +196,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (MASKED) {
-            const int key = k0 + jt * 16 + 4 * kb + i;
+            const int key = k0 + (jt >> 1) * 32 + 8 * kb + (jt & 1) * 4 + i;
             const bool visible = key <= my_pos[b] && (window <= 0 || key > my_pos[b] - window);
             s[b][jt][i] = visible ? s[b][jt][i] : -INFINITY;
           }
@@ -229,28 +241,45 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
       }
 #pragma unroll
       for (int t = 0; t < DTILES; ++t) {
-        const bf16_t* vrow = Vt + (t * 16 + r) * V_ROW + st * 32 + 4 * kb;
-        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+        const bf16x8 a = __builtin_bit_cast(
+            bf16x8, *reinterpret_cast<const uint4*>(Vt + (t * 16 + r) * V_ROW + st * 32 + 8 * kb));
 #pragma unroll
         for (int b = 0; b < RB; ++b) o[b][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[b], o[b][t], 0, 0, 0);
       }
     }
   };
 
-  __syncthreads();                                         // the table entries are in place
-  request(first_tile);
-  for (int k0 = first_tile; k0 < key_end; k0 += BK) {
-    __syncthreads();                                       // the previous tile is consumed
-    publish(k0);
-    __syncthreads();
-    if (k0 + BK < key_end) request(k0 + BK);
+  auto attend_tile = [&](int k0, const bf16_t* tile) {
     if (wave_active && k0 <= wave_last_pos) {
       const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 16 * RB <= n &&
                                (window <= 0 || k0 > wave_last_pos - window);
-      if (all_visible) attend(k0, std::false_type());
-      else attend(k0, std::true_type());
+      if (all_visible) attend(k0, tile, std::false_type());
+      else attend(k0, tile, std::true_type());
+    }
+  };
+  __syncthreads();                                         // the table entries are in place
+  request(first_tile);
+  if (TWO) {
+    publish(first_tile, tiles);
+    if (first_tile + BK < key_end) request(first_tile + BK);
+    __syncthreads();
+    int half = 0;
+    for (int k0 = first_tile; k0 < key_end; k0 += BK, half ^= 1) {
+      // the registers hold the next tile; the other half of the LDS was last read before the barrier
+      if (k0 + BK < key_end) {
+        publish(k0 + BK, tiles + (half ^ 1) * TILE_ELEMS);
+        if (k0 + 2 * BK < key_end) request(k0 + 2 * BK);
+      }
+      attend_tile(k0, tiles + half * TILE_ELEMS);
+      __syncthreads();
+    }
+  } else {
+    for (int k0 = first_tile; k0 < key_end; k0 += BK) {
+      __syncthreads();                                     // the previous tile is consumed
+      publish(k0, tiles);
+      __syncthreads();
+      if (k0 + BK < key_end) request(k0 + BK);
+      attend_tile(k0, tiles);
     }
   }
 
@@ -276,7 +305,7 @@ static int launch_fast(const void* q, int q_stride, const void* k_cache, const v
                        int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s) {
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
-  const size_t lds = ((size_t)FAST_BK * (D + FAST_PAD) + (size_t)D * (FAST_BK + FAST_PAD)) * sizeof(bf16_t) +
+  const size_t lds = (D <= 128 ? 2 : 1) * ((size_t)FAST_BK * (D + FAST_PAD) + (size_t)D * (FAST_BK + FAST_PAD)) * sizeof(bf16_t) +
                      (size_t)table_stride * sizeof(int);
   auto kernel = attn_tile_bf16_kernel<D, RB>;
   static size_t granted = 0;                     // per instantiation
