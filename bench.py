@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine at Qwen3-8B sizes on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16] [--sizes 8b]
 
 Random weights, seeded uniform-random token ids.  A step is one decode step of the
 serving loop (scheduler plan, one batched model step, greedy sampling, events) with
@@ -19,6 +19,16 @@ SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_h
              num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096,
              rms_norm_eps=1e-6, rope_theta=1000000.0, attention_bias=False, tie_word_embeddings=False,
              model_type='qwen3', architectures=['Qwen3ForCausalLM'], hidden_act='silu', eos_token_id=None)
+
+
+# Other layer sizes to measure with --sizes (the default line is always the 8B set above).
+OTHER_SIZES = {
+    '8b': {},
+    '32b': dict(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
+    '0.6b': dict(hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                 tie_word_embeddings=True),
+}
+NAMES = {'8b': 'Qwen3-8B', '32b': 'Qwen3-32B', '0.6b': 'Qwen3-0.6B'}
 
 
 def matrix_params_per_layer(c):
@@ -48,7 +58,8 @@ def main():
     parser.add_argument('--gpus', type=int, default=1)
     parser.add_argument('--steps', type=int, default=64)
     parser.add_argument('--warmup', type=int, default=8)
-    parser.add_argument('--layers', type=int, default=SIZES['num_hidden_layers'])
+    parser.add_argument('--sizes', default='8b', choices=sorted(OTHER_SIZES), help='layer sizes (default: the benchmark\'s)')
+    parser.add_argument('--layers', type=int, default=None, help='fewer layers than the size set has (both numbers are reported)')
     parser.add_argument('--batch', type=int, default=8)
     parser.add_argument('--history', type=int, default=2048)
     parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
@@ -65,7 +76,10 @@ def main():
     from qil_amd import Engine, Qwen3
     from qil_amd.engine import ModelRunner, StepEntry
 
-    config = dict(SIZES, num_hidden_layers=args.layers)
+    sizes = dict(SIZES, **OTHER_SIZES[args.sizes])
+    if args.layers is None:
+        args.layers = sizes['num_hidden_layers']
+    config = dict(sizes, num_hidden_layers=args.layers)
     dtype = getattr(torch, args.dtype)
     element = 2 if args.dtype == 'bfloat16' else 4
     model = Qwen3.from_config(config, seed=0, dtype=dtype, device='cuda:0', on_device=True)
@@ -146,12 +160,13 @@ def main():
     achieved = bytes_read / step_s / 1e9
     flops = prefill_flops(config, args.prefill_tokens)
     line = {
-        'metric': 'decode tok/s at batch 8 (Qwen3-8B sizes, 2048-token histories)', 'value': round(value, 1),
+        'metric': f'decode tok/s at batch {args.batch} ({NAMES[args.sizes]} sizes, {args.history}-token histories)',
+        'value': round(value, 1),
         'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': round(step_s * 1e3, 4), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16' if args.dtype == 'bfloat16' else 'fp32', 'data': 'synthetic',
-        'config': {'model': 'Qwen3-8B sizes, random weights', 'layers': args.layers,
-                   'layers_of_model': SIZES['num_hidden_layers'], 'hidden': config['hidden_size'],
+        'config': {'model': f'{NAMES[args.sizes]} sizes, random weights', 'layers': args.layers,
+                   'layers_of_model': sizes['num_hidden_layers'], 'hidden': config['hidden_size'],
                    'heads': config['num_attention_heads'], 'kv_heads': config['num_key_value_heads'],
                    'head_dim': config['head_dim'], 'intermediate': config['intermediate_size'],
                    'vocab': config['vocab_size'], 'global_batch': args.batch, 'seq_len': args.history,

@@ -15,6 +15,8 @@
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (wave64): lane l supplies A[l % 16][8 (l / 16) .. +7]
 // and B[8 (l / 16) .. +7][l % 16]; it receives D[4 (l / 16) + i][l % 16], i < 4.  A and W rows are
 // both loaded with the same k assignment, so only the D layout matters for correctness.
+#include <algorithm>
+
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -462,12 +464,18 @@ static bool gated_plan(const void* A, const void* W, int M, int inner, int K, in
   for (int c = 8; c >= 1 && !ks; c /= 2)                   // most waves that still leave 16 stages each; else 2 stages
     if (K % (128 * c) == 0 && K / (128 * c) >= (c == 1 ? 2 : 16)) ks = c;
   if (!ks) return false;
+  // Pairs a block: what a CU has to do in all (its blocks one after the other, as many at a time as LDS and
+  // the 12 wave slots allow) over how well its waves keep memory busy (8 or more do).  Ties go to more pairs.
   const int all_pairs = inner / 16;
   int best = 0;
-  long best_cost = 0;
-  for (int pb = GATED_MAX_WAVES / ks; pb >= 1; --pb) {      // rounds of 256 CUs x pairs a block; ties go to more pairs
-    if (gated_lds(M, K, pb * ks) > 156 * 1024) continue;
-    const long blocks = (all_pairs + pb - 1) / pb, cost = (blocks + 255) / 256 * pb;
+  double best_cost = 0;
+  for (int pb = GATED_MAX_WAVES / ks; pb >= 1; --pb) {
+    const size_t lds = gated_lds(M, K, pb * ks);
+    if (lds > 156 * 1024) continue;
+    const long resident = std::max<long>(1, std::min<long>((160 * 1024) / lds, GATED_MAX_WAVES / (pb * ks)));
+    const long blocks = (all_pairs + pb - 1) / pb, per_cu = (blocks + 255) / 256;
+    const long together = std::min(resident, per_cu), rounds = (per_cu + together - 1) / together;
+    const double cost = (double)rounds * pb * 8.0 / (double)std::min<long>(8, together * pb * ks);
     if (!best || cost < best_cost) { best = pb; best_cost = cost; }
   }
   if (!best) return false;
