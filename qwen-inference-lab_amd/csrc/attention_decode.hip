@@ -27,7 +27,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define DEC_MAX_WAVES 8                                    // waves of a block; each takes every waves-th 32-key step
 
-template <int DMAX>
+template <int DMAX, bool PAIRS>
 __global__ void __launch_bounds__(DEC_MAX_WAVES * QIL_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
@@ -67,32 +67,41 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 
   const int first_step = begin / 32;                       // 32-key steps, absolute numbering
   const int last_step = (end - 1) / 32;
-  for (int step = first_step + wave; step <= last_step; step += waves) {
+  // What one 32-key step needs from memory: the K rows of both 16-key sub-tiles and the V^T fragments
+  // of every dim tile, found through three entries of the block table.
+  struct StepData {
+    uint4 k[2][QFRAGS];
+    uint4 v[DTILES];                                        // V^T[dim 16 t + r][keys 8 kb .. 8 kb + 7]: 16 bytes of one page row
+  };
+  auto look_up = [&](int step, int (&page)[3]) {
     const int k0 = step * 32;
-    // ---- loads first: K rows of both 16-key sub-tiles, then the V^T fragments of every dim tile
-    uint4 kraw[2][QFRAGS];
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
+    for (int jt = 0; jt < 2; ++jt)
       // row r of sub-tile jt is key 8 (r / 4) + 4 jt + r % 4 of the step, so that a lane's eight
       // scores (rows 4 kb + i of both sub-tiles) are the eight consecutive keys 8 kb .. 8 kb + 7
-      const int key = min(k0 + 8 * (r >> 2) + 4 * jt + (r & 3), ctx - 1);   // clamped: an invisible key's score is replaced below
-      const size_t page = table[key / page_size];
-      const bf16_t* krow = k_cache + ((page * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d;
+      page[jt] = table[min(k0 + 8 * (r >> 2) + 4 * jt + (r & 3), ctx - 1) / page_size];   // clamped: an invisible key's score is replaced
+    page[2] = table[(min(k0 + 8 * kb, ctx - 1) & ~7) / page_size];
+  };
+  auto request = [&](int step, const int (&page)[3], StepData& data) {
+    const int k0 = step * 32;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+      const int key = min(k0 + 8 * (r >> 2) + 4 * jt + (r & 3), ctx - 1);
+      const bf16_t* krow = k_cache + (((size_t)page[jt] * kv_heads + kvh) * page_size + (key % page_size)) * (size_t)d;
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks) {
         const int dim = ks * 32 + kb * 8;
-        kraw[jt][ks] = (ks * 32 < d && dim < d) ? *reinterpret_cast<const uint4*>(krow + dim) : make_uint4(0, 0, 0, 0);
+        data.k[jt][ks] = (ks * 32 < d && dim < d) ? *reinterpret_cast<const uint4*>(krow + dim) : make_uint4(0, 0, 0, 0);
       }
     }
-    uint4 vraw[DTILES];                                     // V^T[dim 16 t + r][keys 8 kb .. 8 kb + 7]: 16 bytes of one page row
-    {
-      const int key = min(k0 + 8 * kb, ctx - 1) & ~7;
-      const size_t page = table[key / page_size];
-      const bf16_t* vbase = v_cache + (page * kv_heads + kvh) * (size_t)d * page_size + (key % page_size);
+    const int key = min(k0 + 8 * kb, ctx - 1) & ~7;
+    const bf16_t* vbase = v_cache + ((size_t)page[2] * kv_heads + kvh) * (size_t)d * page_size + (key % page_size);
 #pragma unroll
-      for (int t = 0; t < DTILES; ++t)
-        vraw[t] = t < dt ? *reinterpret_cast<const uint4*>(vbase + (size_t)(t * 16 + r) * page_size) : make_uint4(0, 0, 0, 0);
-    }
+    for (int t = 0; t < DTILES; ++t)
+      data.v[t] = t < dt ? *reinterpret_cast<const uint4*>(vbase + (size_t)(t * 16 + r) * page_size) : make_uint4(0, 0, 0, 0);
+  };
+  auto attend = [&](int step, const StepData& data) {
+    const int k0 = step * 32;
     // ---- scores
     f32x4 s[2];
 #pragma unroll
@@ -100,7 +109,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks)
-        if (ks * 32 < d) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kraw[jt][ks]), qb[ks], acc, 0, 0, 0);
+        if (ks * 32 < d) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, data.k[jt][ks]), qb[ks], acc, 0, 0, 0);
       s[jt] = acc;
     }
     float mx = -INFINITY;
@@ -144,12 +153,37 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 #pragma unroll
     for (int t = 0; t < DTILES; ++t) {
       if (t < dt) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vraw[t].x & mask[0], vraw[t].y & mask[1],
-                                                                vraw[t].z & mask[2], vraw[t].w & mask[3]));
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(data.v[t].x & mask[0], data.v[t].y & mask[1],
+                                                                data.v[t].z & mask[2], data.v[t].w & mask[3]));
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
         o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[t], 0, 0, 0);
       }
+    }
+  };
+  if (PAIRS) {
+    // Two of the wave's steps at a time: both steps' table entries, then both steps' K and V, then the
+    // arithmetic; a wave waits for memory twice per pair instead of twice per step.  (Twice the
+    // registers: for launches that leave a CU's register file to one block.)
+    for (int step = first_step + wave; step <= last_step; step += 2 * waves) {
+      const int second = step + waves;
+      const bool two = second <= last_step;
+      int page_a[3], page_b[3];
+      StepData a, b;
+      look_up(step, page_a);
+      if (two) look_up(second, page_b);
+      request(step, page_a, a);
+      if (two) request(second, page_b, b);
+      attend(step, a);
+      if (two) attend(second, b);
+    }
+  } else {
+    for (int step = first_step + wave; step <= last_step; step += waves) {
+      int page[3];
+      StepData data;
+      look_up(step, page);
+      request(step, page, data);
+      attend(step, data);
     }
   }
 
@@ -198,12 +232,13 @@ extern "C" int qil_attn_decode_takes(int heads, int kv_heads, int d, int page_si
 
 // Partial results in the layout of the row kernel (acc [rows, heads, parts, d], then m, then l);
 // the caller runs the row kernel's merge when parts > 1.  P must be a multiple of 32; a block has
-// `waves` waves (at most 8), best one or two 32-key steps of P for each.
+// `waves` waves (at most 8), best one or two 32-key steps of P for each.  pairs != 0: a wave loads two of
+// its steps at a time (twice the registers; for launches of at most one block a CU).
 extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* block_tables, int table_stride, const int* row_seq, const int* positions,
                                const int* row_index, void* workspace, void* out, int rows, int heads, int kv_heads,
                                int d, int page_size, int window, float scale, int P, int parts, int waves,
-                               hipStream_t s) {
+                               int pairs, hipStream_t s) {
   if (rows == 0) return 0;
   if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || P % 32 || P < 32 || parts < 1 || parts > 65535 ||
       kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES)
@@ -215,7 +250,12 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
   const size_t lds = (size_t)waves * g * (d + 2) * sizeof(float);
   dim3 grid(rows, kv_heads, parts);
 #define QIL_DEC_CASE(DMAX)                                                                                          \
-  hipLaunchKernelGGL(attn_decode_kernel<DMAX>, grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
+  if (pairs)                                                                                                        \
+    hipLaunchKernelGGL((attn_decode_kernel<DMAX, true>), grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
+                     (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
+                     row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts);   \
+  else                                                                                                              \
+  hipLaunchKernelGGL((attn_decode_kernel<DMAX, false>), grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
                      (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
                      row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts)
   if (d <= 64) QIL_DEC_CASE(64);

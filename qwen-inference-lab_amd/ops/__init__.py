@@ -27,6 +27,8 @@ DECODE_WAVES = 8
 DECODE_MIN_PART = 256
 # Most keys of a block.
 DECODE_MAX_PART = 8192
+# Launches of at most this many blocks (one a CU) let a wave load two of its steps at a time.
+DECODE_PAIRS_BLOCKS = 256
 
 
 class UnsupportedShape(ValueError):
@@ -341,7 +343,9 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             _check(lib.qil_attn_decode(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                        block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                        _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
-                                       window_arg, float(scale), part, parts, DECODE_WAVES, _stream()), 'attn_decode')
+                                       window_arg, float(scale), part, parts, DECODE_WAVES,
+                                       int(rows * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= 128), _stream()),
+                   'attn_decode')
             if unmerged and parts > 1 and single_rows is None:
                 return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
                                 part=part, parts=parts)

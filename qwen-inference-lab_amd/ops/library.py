@@ -148,7 +148,7 @@ def _declare(lib):
     lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
     lib.qil_attn_decode_takes.restype = i
-    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, p]
     lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_splits.argtypes = [i, i, i]

@@ -344,6 +344,176 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     assert not torch.allclose(last[0], whole['a'][-1], atol=1e-3)
 
 
+def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
+    """Parts the framework does not have, defined here and used without a change to its files: a feed-forward
+    that routes each token to one of three experts (router logits in float32), and a position encoding that
+    rotates half of each head by scaled positions.  They sit beside the framework's attention run with
+    options Qwen3 never uses (bias, no q/k norm, a window, a scale of its own).  Checked against a float64
+    restatement of the same model written here, whole and in pieces, through the decode graph too."""
+    from dataclasses import dataclass
+    from safetensors.torch import load_file
+    from qil_amd import ops
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.parts import (Attention, FeedForward, ParamSpec, PositionEncoding, Rotation, RMSNorm, PreNormBlock,
+                               Embedding, LMHead, CausalLM, ScheduleEntry)
+    from qil_amd.registry import register_architecture
+    from qil_amd.weights import write_random_model, load_model
+
+    class ScaledHalfRotary(PositionEncoding):
+        def __init__(self, head_dim, theta, factor, max_positions, device):
+            super().__init__()
+            self.rot, self.theta, self.factor, self.max_positions, self.device = head_dim // 2, theta, factor, max_positions, device
+            self.tables = None
+
+        def rotation(self):                                  # called in every step: the tables are made once
+            if self.tables is None:
+                inv_freq = 1.0 / self.theta ** (torch.arange(0, self.rot, 2, dtype=torch.float32) / self.rot)
+                angles = (torch.arange(self.max_positions, dtype=torch.float32) / self.factor)[:, None] * inv_freq
+                self.tables = Rotation(angles.cos().to(self.device).contiguous(), angles.sin().to(self.device).contiguous(),
+                                       self.rot)
+            return self.tables
+
+    class Top1Experts(FeedForward):
+        def __init__(self, width, inner, experts, dtype):
+            super().__init__()
+            self.width, self.inner, self.experts, self.dtype = width, inner, experts, dtype
+
+        def param_specs(self):
+            specs = {'router.weight': ParamSpec((self.experts, self.width))}
+            for e in range(self.experts):
+                specs[f'experts.{e}.gate_up.weight'] = ParamSpec((2 * self.inner, self.width))
+                specs[f'experts.{e}.down.weight'] = ParamSpec((self.width, self.inner))
+            return specs
+
+        def forward(self, h):
+            choice = ops.linear(h, self.p['router.weight'], None, out_dtype=torch.float32).argmax(dim=-1)
+            out = torch.zeros(h.shape, dtype=self.dtype, device=h.device)
+            for e in range(self.experts):                    # every expert on every token, then a select: no host decision
+                y = ops.linear(ops.gated_linear(h, self.p[f'experts.{e}.gate_up.weight'], self.dtype),
+                               self.p[f'experts.{e}.down.weight'], None)
+                out = torch.where((choice == e)[:, None], y, out)
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        layers: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        inner: int
+        experts: int
+        window: int
+        eps: float = 1e-5
+        theta: float = 500.0
+        factor: float = 2.0
+        max_position_embeddings: int = 128
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+        def to_dict(self):
+            return dict(self.__dict__, architectures=['ToyRoutedLM'], model_type='toy_routed')
+
+    def build(c, *, dtype, device):
+        embedding = Embedding(c.vocab_size, c.hidden_size)
+        position = ScaledHalfRotary(c.head_dim, c.theta, c.factor, c.max_position_embeddings, device)
+        blocks = [PreNormBlock(mixer_norm=RMSNorm(c.hidden_size, c.eps),
+                               mixer=Attention(width=c.hidden_size, heads=c.heads, kv_heads=c.kv_heads, head_dim=c.head_dim,
+                                               bias=True, qk_norm_eps=None, scale=1.7 * c.head_dim ** -0.5,
+                                               position=position, window=c.window, dtype=dtype),
+                               ffn_norm=RMSNorm(c.hidden_size, c.eps),
+                               ffn=Top1Experts(c.hidden_size, c.inner, c.experts, dtype), dtype=dtype)
+                  for _ in range(c.layers)]
+        final_norm, head = RMSNorm(c.hidden_size, c.eps), LMHead(c.vocab_size, c.hidden_size)
+        names = {'embed.weight': (embedding, 'weight'), 'norm.weight': (final_norm, 'weight'), 'head.weight': (head, 'weight')}
+        for i, block in enumerate(blocks):
+            for prefix, part in block.parts().items():
+                for local in part.param_specs():
+                    names[f'layers.{i}.{prefix}.{local}'] = (part, local)
+        return CausalLM(config=c, embedding=embedding, blocks=blocks, schedule=[ScheduleEntry(i) for i in range(len(blocks))],
+                        final_norm=final_norm, head=head, names=names, dtype=dtype, device=device)
+
+    register_architecture('ToyRoutedLM', model_type='toy_routed', config_class=ToyConfig, build=build, replace=True)
+    data = dict(architectures=['ToyRoutedLM'], model_type='toy_routed', vocab_size=150, hidden_size=56, layers=2, heads=6,
+                kv_heads=3, head_dim=16, inner=48, experts=3, window=7)
+    folder = write_random_model(tmp_path / 'routed', data, seed=9, dtype=torch.float32)
+    w = {k: v.double() for k, v in load_file(str(folder / 'model.safetensors')).items()}
+    c = ToyConfig.from_dict(data)
+
+    def expected(tokens):
+        """The same model in float64, whole sequence, no cache."""
+        n, d, g = len(tokens), c.head_dim, c.heads // c.kv_heads
+        x = w['embed.weight'][tokens]
+        norm = lambda v, weight: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + c.eps) * weight
+        rot = d // 2
+        inv_freq = 1.0 / c.theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot)
+        angles = ((torch.arange(n, dtype=torch.float32) / c.factor)[:, None] * inv_freq).double()
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+
+        def rotate(t):                                       # [n, heads, d]: pairs (i, i + rot / 2) of the first rot dims
+            a, b, rest = t[..., :rot // 2], t[..., rot // 2:rot], t[..., rot:]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, rest], dim=-1)
+        margins = []
+        for i in range(c.layers):
+            pre = f'layers.{i}.'
+            h = norm(x, w[pre + 'mixer_norm.weight'])
+            q = (h @ w[pre + 'mixer.q_proj.weight'].t() + w[pre + 'mixer.q_proj.bias']).view(n, c.heads, d)
+            k = (h @ w[pre + 'mixer.k_proj.weight'].t() + w[pre + 'mixer.k_proj.bias']).view(n, c.kv_heads, d)
+            v = (h @ w[pre + 'mixer.v_proj.weight'].t() + w[pre + 'mixer.v_proj.bias']).view(n, c.kv_heads, d)
+            q, k = rotate(q), rotate(k).repeat_interleave(g, dim=1)
+            score = torch.einsum('qhd,khd->hqk', q, k) * (1.7 * d ** -0.5)
+            at = torch.arange(n)
+            visible = (at[None, :] <= at[:, None]) & (at[None, :] > at[:, None] - c.window)
+            score = score.masked_fill(~visible, float('-inf')).softmax(-1)
+            mixed = torch.einsum('hqk,khd->qhd', score, v.repeat_interleave(g, dim=1)).reshape(n, -1)
+            x = x + mixed @ w[pre + 'mixer.o_proj.weight'].t() + w[pre + 'mixer.o_proj.bias']
+            h = norm(x, w[pre + 'ffn_norm.weight'])
+            router = h @ w[pre + 'ffn.router.weight'].t()
+            top = router.topk(2, dim=-1).values
+            margins.append((top[:, 0] - top[:, 1]).min().item())
+            y = torch.zeros_like(x)
+            for e in range(c.experts):
+                both = h @ w[pre + f'ffn.experts.{e}.gate_up.weight'].t()
+                act = torch.nn.functional.silu(both[:, :c.inner]) * both[:, c.inner:]
+                y = torch.where((router.argmax(-1) == e)[:, None], act @ w[pre + f'ffn.experts.{e}.down.weight'].t(), y)
+            x = x + y
+        return norm(x, w['norm.weight']) @ w['head.weight'].t(), min(margins)
+
+    prompts = prompts_for(data, [23, 9], 3)
+    wanted = {}
+    for name, tokens in zip('ab', prompts):
+        wanted[name], margin = expected(tokens)
+        assert margin > 1e-3, 'a router decision of this test is too close to call in float32: pick another seed'
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+
+    def run(cuts):
+        runner = ModelRunner(model, num_pages=6, page_size=8, max_requests=2)
+        for name in 'ab':
+            runner.admit(name)
+        got, at = {'a': [], 'b': []}, {'a': 0, 'b': 0}
+        for sizes in cuts:
+            entries = [StepEntry(name, tuple(tokens[at[name]:at[name] + size]), tuple(range(size)))
+                       for name, size, tokens in zip('ab', sizes, prompts) if size]
+            logits = runner.step(entries)
+            row = 0
+            for entry in entries:
+                got[entry.request].append(logits[row:row + len(entry.tokens)])
+                row += len(entry.tokens)
+                at[entry.request] += len(entry.tokens)
+        return {name: torch.cat(parts) for name, parts in got.items()}, runner
+
+    whole, _ = run([(23, 9)])
+    pieces, runner = run([(14, 3), (2, 1), (1, 1), (1, 1), (1, 1), (4, 2)])     # three steps of single tokens: the graph
+    assert runner.graphs is None or runner.graphs.replays >= 3
+    assert runner.cache.kv_groups[0]['pool'].window == 7, 'the window reached the page pool'
+    for name in 'ab':
+        torch.testing.assert_close(whole[name].double().cpu(), wanted[name], atol=2e-5, rtol=2e-4)
+        torch.testing.assert_close(pieces[name].double().cpu(), wanted[name], atol=2e-5, rtol=2e-4)
+
+
 # ------------------------------------------------------------------------------- real layer sizes
 
 REAL = {
