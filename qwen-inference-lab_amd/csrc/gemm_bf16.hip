@@ -155,7 +155,7 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
 // fragments.  The 16-byte pieces of a row are stored at piece ^ row, so the writes (16 lanes, one
 // row) and the fragment reads (16 lanes, 16 rows, one logical piece) both spread over all banks.
 // LDS operations of one wave complete in program order, so the buffer needs no barrier.
-// Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
+// Takes M <= 64, K a multiple of 128 per split, 16-byte aligned operands, no bias.
 #define LINES_WAVES 8
 
 // A given as the unmerged partial results of split-context attention (attention_rows.hip,
@@ -213,14 +213,15 @@ __device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
                     pack_bf16(numer[4] / denom, numer[5] / denom), pack_bf16(numer[6] / denom, numer[7] / denom));
 }
 
-template <typename OUT, bool MERGE>
+// MT: 16-row tiles of A (M <= 16 MT); every W fragment read from the buffer serves MT products.
+template <typename OUT, bool MERGE, int MT>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
 gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const bf16_t* __restrict__ W,
                        OUT* __restrict__ C, int M, int N, int K, int cols_per_split) {
-  extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
+  extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16 MT][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
+  const int a_rows = MT > 1 ? 16 * MT : M <= 8 ? 8 : 16;   // rows of A kept; the others multiply as zeros
   const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
   const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
   const int row_width = cols_per_split + GEMM_LDS_PAD;
@@ -259,7 +260,9 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   request(w2, 2);
   __syncthreads();
 
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const bool a_live = r < a_rows;
   const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + kb * 8;
   auto pass = [&](const u32x4 (&stage_w)[4]) {             // registers -> buffer
@@ -272,10 +275,13 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
-      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
-      if (!a_live) a = (u32x4){0, 0, 0, 0};
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
-                                                    0, 0);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        u32x4 a = *reinterpret_cast<const u32x4*>(a_row + t * 16 * row_width + at + s4 * 32);
+        if (MT == 1 && !a_live) a = (u32x4){0, 0, 0, 0};
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                         acc[t], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -294,29 +300,32 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   if (left > 4) { pass(w1); multiply(stage + 4); }
   OUT* out = C + (size_t)split * M * N;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = 4 * kb + i, n = n0 + r;
-    if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[i]);
-  }
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = t * 16 + 4 * kb + i, n = n0 + r;
+      if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[t][i]);
+    }
 }
 
 static size_t lines_lds(int M, int K, int splits) {
-  return ((size_t)(M <= 8 ? 8 : 16) * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
+  const int rows = M <= 8 ? 8 : M <= 16 ? 16 : M <= 32 ? 32 : 64;
+  return ((size_t)rows * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
 }
 
 // Whether the whole-line kernel takes the product with this many splits.
 static bool lines_takes(const void* A, const void* W, const float* bias, int M, int N, int K, int splits) {
-  if (bias || M > 16 || N < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH ||
+  if (bias || M > 64 || N < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH ||
       (((uintptr_t)A | (uintptr_t)W) % 16))
     return false;
   return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
 }
 
-template <typename OUT, bool MERGE = false>
-static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
-                        UnmergedA unmerged = UnmergedA()) {
+template <typename OUT, bool MERGE, int MT>
+static int launch_lines_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
+                              UnmergedA unmerged) {
   const size_t lds = lines_lds(M, K, splits);
-  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE>;
+  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE, MT>;
   static size_t granted = 0;                              // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -326,6 +335,15 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
   dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
   hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, unmerged, W, C, M, N, K, K / splits);
   return 0;
+}
+
+template <typename OUT, bool MERGE = false>
+static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
+                        UnmergedA unmerged = UnmergedA()) {
+  if (M <= 16) return launch_lines_tiles<OUT, MERGE, 1>(A, W, C, M, N, K, splits, s, unmerged);
+  if (MERGE) return -1;                                    // the merge is made for the few rows of decode steps
+  if (M <= 32) return launch_lines_tiles<OUT, false, 2>(A, W, C, M, N, K, splits, s, unmerged);
+  return launch_lines_tiles<OUT, false, 4>(A, W, C, M, N, K, splits, s, unmerged);
 }
 
 // ---------------------------------------------------------------------------------------------------
