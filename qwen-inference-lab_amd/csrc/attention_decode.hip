@@ -21,15 +21,41 @@
 //
 // Takes page_size % 8 == 0, d % 16 == 0, d <= 256, g <= 16; other sizes go to the row kernel.
 #include "common.h"
+#include "qk_math.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define DEC_MAX_WAVES 8                                    // waves of a block; each takes every waves-th 32-key step
 
-template <int DMAX, bool PAIRS>
+// FUSED: the queries do not come from memory but from the partial sums of the q/k/v product, with the
+// head norm and the rotation made here (the arithmetic of qk_rope.hip, shared through qk_math.h); and the
+// wave that meets the row's own position makes the new key and value the same way, writes them into the
+// pages and uses them from its registers.  One kernel less per layer in a decode step.
+struct FusedQKV {
+  const float* qkv;                                        // [splits][rows][(heads + 2 kv_heads) d] partial sums
+  size_t split_stride;
+  int splits;
+  const float* q_weight;                                   // null: no head norm
+  const float* k_weight;
+  float eps;
+  const float* cos_table;                                  // null: no rotation
+  const float* sin_table;
+  int rot;
+  int writes;                                              // 0: the cache belongs to another layer, which wrote it
+};
+
+__device__ __forceinline__ uint4 pack8(const float* v) {
+  return make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+}
+__device__ __forceinline__ uint4 shuffle4(uint4 v, int source) {
+  return make_uint4(__shfl(v.x, source, QIL_WAVE), __shfl(v.y, source, QIL_WAVE), __shfl(v.z, source, QIL_WAVE),
+                    __shfl(v.w, source, QIL_WAVE));
+}
+
+template <int DMAX, bool PAIRS, bool FUSED>
 __global__ void __launch_bounds__(DEC_MAX_WAVES * QIL_WAVE)
-attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                    const int* __restrict__ row_seq, const int* __restrict__ positions,
                    const int* __restrict__ row_index, float* __restrict__ part_acc, float* __restrict__ part_m,
@@ -50,23 +76,19 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   const int dt = d / 16;
   const int* table = block_tables + (size_t)row_seq[row] * table_stride;
 
-  // Q fragments: B operand, column r = head kvh * g + r
+  const int first_step = begin / 32;                       // 32-key steps, absolute numbering
+  const int last_step = (end - 1) / 32;
+
+  // Q fragments: B operand, column r = head kvh * g + r (filled below, after the first loads are on their way)
   bf16x8 qb[QFRAGS];
-#pragma unroll
-  for (int ks = 0; ks < QFRAGS; ++ks) {
-    const int dim = ks * 32 + kb * 8;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    if (r < g && dim < d) raw = *reinterpret_cast<const uint4*>(q + (size_t)row * q_stride + (size_t)(kvh * g + r) * d + dim);
-    qb[ks] = __builtin_bit_cast(bf16x8, raw);
-  }
+  uint4 new_k = make_uint4(0, 0, 0, 0), new_v = make_uint4(0, 0, 0, 0);   // FUSED: chunk lane % (DMAX / 8) of the new key / value
+  bool owner = false;                                      // FUSED: this wave meets the row's own position
 
   float m = -INFINITY, l = 0.f;
   f32x4 o[DTILES];
 #pragma unroll
   for (int t = 0; t < DTILES; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int first_step = begin / 32;                       // 32-key steps, absolute numbering
-  const int last_step = (end - 1) / 32;
   // What one 32-key step needs from memory: the K rows of both 16-key sub-tiles and the V^T fragments
   // of every dim tile, found through three entries of the block table.
   struct StepData {
@@ -100,8 +122,37 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     for (int t = 0; t < DTILES; ++t)
       data.v[t] = t < dt ? *reinterpret_cast<const uint4*>(vbase + (size_t)(t * 16 + r) * page_size) : make_uint4(0, 0, 0, 0);
   };
-  auto attend = [&](int step, const StepData& data) {
+  auto attend = [&](int step, StepData& data) {
     const int k0 = step * 32;
+    if constexpr (FUSED) {
+      if (owner && step == (pos >> 5)) {                   // the new key and value come from this wave's registers
+        const int local = pos & 31;                          // key 8 (rr / 4) + 4 jt + rr % 4 of the step
+        const int jt_new = (local >> 2) & 1, rr = ((local >> 3) << 2) | (local & 3);
+#pragma unroll
+        for (int ks = 0; ks < QFRAGS; ++ks) {
+          const uint4 piece = shuffle4(new_k, 4 * ks + kb);
+#pragma unroll
+          for (int jt = 0; jt < 2; ++jt)
+            if (r == rr && jt == jt_new) data.k[jt][ks] = piece;
+        }
+        const int j = local & 7;                             // element of the lanes with kb == local / 8
+#pragma unroll
+        for (int t = 0; t < DTILES; ++t) {
+          const uint4 piece = shuffle4(new_v, 2 * t + (r >> 3));             // chunk of dim 16 t + r
+          const int e = r & 7;
+          const uint32_t word = (e >> 1) == 0 ? piece.x : (e >> 1) == 1 ? piece.y : (e >> 1) == 2 ? piece.z : piece.w;
+          const uint32_t value = (word >> ((e & 1) * 16)) & 0xffffu;
+          if (kb == (local >> 3)) {
+            const uint32_t shift = (j & 1) * 16, keep = ~(0xffffu << shift), put = value << shift;
+            uint32_t w[4] = {data.v[t].x, data.v[t].y, data.v[t].z, data.v[t].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (i == (j >> 1)) w[i] = (w[i] & keep) | put;
+            data.v[t] = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        }
+      }
+    }
     // ---- scores
     f32x4 s[2];
 #pragma unroll
@@ -161,29 +212,94 @@ attn_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
       }
     }
   };
+  auto make_queries = [&]() {
+    if constexpr (FUSED) {
+      constexpr int TG = DMAX / 8, HPP = QIL_WAVE / TG;      // lanes of a head (8 elements each), heads a pass
+      const int total_heads = heads + 2 * kv_heads;
+      const int chunk = lane % TG, sub = lane / TG;
+      // the block's waves share the heads (HPP of them a wave and pass); the queries meet in LDS
+      uint4* shared_q = reinterpret_cast<uint4*>(lds);       // [g][TG] chunks; the end of the kernel uses the LDS again
+      for (int base = wave * HPP; base < g; base += waves * HPP) {
+        float x[8];
+        const int head = kvh * g + min(base + sub, g - 1);   // lanes past the group repeat its last head
+        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + head) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        norm_rope8<bf16_t>(x, chunk, TG, fused.q_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot);
+        if (base + sub < g) shared_q[(base + sub) * TG + chunk] = pack8(x);
+      }
+      owner = fused.writes && pos >= begin && pos < end && wave == ((pos >> 5) - first_step) % waves;
+      if (owner) {                                           // wave-uniform
+        float x[8];
+        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kvh) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        norm_rope8<bf16_t>(x, chunk, TG, fused.k_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot);
+        new_k = pack8(x);
+        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kv_heads + kvh) * DMAX + chunk * 8, fused.splits,
+                       fused.split_stride, x);
+        new_v = pack8(x);
+        if (sub == 0) {                                      // into the pages (qil/cache.py:79-82)
+          const size_t page = table[pos / page_size];
+          const int offset = pos % page_size;
+          bf16_t* k_row = const_cast<bf16_t*>(k_cache) + ((page * kv_heads + kvh) * page_size + offset) * (size_t)DMAX;
+          *reinterpret_cast<uint4*>(k_row + chunk * 8) = new_k;
+          bf16_t* column = const_cast<bf16_t*>(v_cache) + ((page * kv_heads + kvh) * (size_t)DMAX + chunk * 8) * page_size + offset;
+          const uint32_t words[4] = {new_v.x, new_v.y, new_v.z, new_v.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) column[(size_t)e * page_size] = (bf16_t)(words[e >> 1] >> ((e & 1) * 16));
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < QFRAGS; ++ks)                    // fragment ks of head r = chunk 4 ks + kb of that head
+        qb[ks] = __builtin_bit_cast(bf16x8, r < g ? shared_q[r * TG + 4 * ks + kb] : make_uint4(0, 0, 0, 0));
+      __syncthreads();                                       // the LDS is free again
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < QFRAGS; ++ks) {
+        const int dim = ks * 32 + kb * 8;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (r < g && dim < d) raw = *reinterpret_cast<const uint4*>(q + (size_t)row * q_stride + (size_t)(kvh * g + r) * d + dim);
+        qb[ks] = __builtin_bit_cast(bf16x8, raw);
+      }
+    }
+  };
+  // The loads of a wave's first step (or pair of steps) go out before its queries are made, so that the
+  // two waits overlap; later steps are loaded when the step before is done.
   if (PAIRS) {
     // Two of the wave's steps at a time: both steps' table entries, then both steps' K and V, then the
     // arithmetic; a wave waits for memory twice per pair instead of twice per step.  (Twice the
     // registers: for launches that leave a CU's register file to one block.)
-    for (int step = first_step + wave; step <= last_step; step += 2 * waves) {
-      const int second = step + waves;
-      const bool two = second <= last_step;
-      int page_a[3], page_b[3];
-      StepData a, b;
+    int step = first_step + wave;
+    int page_a[3], page_b[3];
+    StepData a, b;
+    auto load_pair = [&]() {
       look_up(step, page_a);
-      if (two) look_up(second, page_b);
+      if (step + waves <= last_step) look_up(step + waves, page_b);
       request(step, page_a, a);
-      if (two) request(second, page_b, b);
+      if (step + waves <= last_step) request(step + waves, page_b, b);
+    };
+    if (step <= last_step) load_pair();
+    make_queries();
+    while (step <= last_step) {
       attend(step, a);
-      if (two) attend(second, b);
+      if (step + waves <= last_step) attend(step + waves, b);
+      step += 2 * waves;
+      if (step <= last_step) load_pair();
     }
   } else {
-    for (int step = first_step + wave; step <= last_step; step += waves) {
-      int page[3];
-      StepData data;
+    int step = first_step + wave;
+    int page[3];
+    StepData data;
+    if (step <= last_step) {
       look_up(step, page);
       request(step, page, data);
+    }
+    make_queries();
+    while (step <= last_step) {
       attend(step, data);
+      step += waves;
+      if (step <= last_step) {
+        look_up(step, page);
+        request(step, page, data);
+      }
     }
   }
 
@@ -249,18 +365,70 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
   float* l = m ? m + (size_t)rows * heads * parts : nullptr;
   const size_t lds = (size_t)waves * g * (d + 2) * sizeof(float);
   dim3 grid(rows, kv_heads, parts);
+  const FusedQKV none = {};
+#define QIL_DEC_LAUNCH(DMAX, PAIRS, FUSED, FIELDS)                                                                  \
+  hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, FUSED>), grid, dim3(waves * QIL_WAVE), lds, s, FIELDS,         \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
+                     table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
+                     page_size, window, scale, P, parts)
 #define QIL_DEC_CASE(DMAX)                                                                                          \
-  if (pairs)                                                                                                        \
-    hipLaunchKernelGGL((attn_decode_kernel<DMAX, true>), grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
-                     (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
-                     row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts);   \
-  else                                                                                                              \
-  hipLaunchKernelGGL((attn_decode_kernel<DMAX, false>), grid, dim3(waves * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride,          \
-                     (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_stride, row_seq, positions, \
-                     row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d, page_size, window, scale, P, parts)
+  if (pairs) QIL_DEC_LAUNCH(DMAX, true, false, none);                                                               \
+  else QIL_DEC_LAUNCH(DMAX, false, false, none)
   if (d <= 64) QIL_DEC_CASE(64);
   else if (d <= 128) QIL_DEC_CASE(128);
   else QIL_DEC_CASE(256);
 #undef QIL_DEC_CASE
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// 1 if the fused kernel (queries, new key and new value made from the q/k/v product's partial sums) takes
+// the sizes: a head of exactly 64 or 128 elements (256 would not fit the registers), a rotated width the
+// vector kernel of qk_rope.hip takes.
+extern "C" int qil_attn_decode_fused_takes(int heads, int kv_heads, int d, int page_size, int rot) {
+  if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || !(d == 64 || d == 128)) return 0;
+  const int half_chunks = rot >> 4;
+  return rot == 0 || (rot <= d && rot % 16 == 0 && (half_chunks & (half_chunks - 1)) == 0);
+}
+
+// qil_attn_decode with qkv [splits][rows][(heads + 2 kv_heads) d] float32 partial sums in the place of q; the
+// rows are the step's rows 0 .. rows-1 (no row index).  q_weight, k_weight: both or neither; cos/sin: both
+// or neither, [positions][rot / 2].  writes != 0: the new keys and values go into the caches at the rows'
+// positions (the page comes from the block table).
+extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* q_weight, const float* k_weight,
+                                     float eps, const float* cos_table, const float* sin_table, int rot, int writes,
+                                     void* k_cache, void* v_cache, const int* block_tables, int table_stride,
+                                     const int* row_seq, const int* positions, void* workspace, void* out, int rows,
+                                     int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
+                                     int parts, int waves, int pairs, hipStream_t s) {
+  if (rows == 0) return 0;
+  if (!qil_attn_decode_fused_takes(heads, kv_heads, d, page_size, cos_table ? rot : 0) || P % 32 || P < 32 ||
+      parts < 1 || parts > 65535 || kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES || splits < 1 ||
+      (q_weight == nullptr) != (k_weight == nullptr) || (cos_table == nullptr) != (sin_table == nullptr) ||
+      (((uintptr_t)qkv | (uintptr_t)q_weight | (uintptr_t)k_weight | (uintptr_t)cos_table | (uintptr_t)sin_table |
+        (uintptr_t)k_cache) % 16))
+    return -1;
+  const int g = heads / kv_heads;
+  float* acc = (float*)workspace;
+  float* m = acc ? acc + (size_t)rows * heads * parts * d : nullptr;
+  float* l = m ? m + (size_t)rows * heads * parts : nullptr;
+  const size_t lds = (size_t)waves * g * (d + 2) * sizeof(float);
+  dim3 grid(rows, kv_heads, parts);
+  FusedQKV fused;
+  fused.qkv = qkv;
+  fused.split_stride = (size_t)rows * (heads + 2 * kv_heads) * d;
+  fused.splits = splits;
+  fused.q_weight = q_weight; fused.k_weight = k_weight; fused.eps = eps;
+  fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rot = cos_table ? rot : 0;
+  fused.writes = writes;
+  const void* q = nullptr;
+  const int q_stride = 0;
+  const int* row_index = nullptr;
+#define QIL_DEC_CASE(DMAX)                                                                                          \
+  if (pairs) QIL_DEC_LAUNCH(DMAX, true, true, fused);                                                               \
+  else QIL_DEC_LAUNCH(DMAX, false, true, fused)
+  if (d == 64) QIL_DEC_CASE(64);
+  else QIL_DEC_CASE(128);
+#undef QIL_DEC_CASE
+#undef QIL_DEC_LAUNCH
   QIL_RETURN_LAUNCH_STATUS();
 }

@@ -1,0 +1,93 @@
+// Eight consecutive elements of a head at a time: the sum of a product's partial results, the head's
+// RMSNorm and the rotation by position, as the vector kernel of qk_rope.hip and the fused decode
+// attention (attention_decode.hip) both do them.  One source for both, so that a query or key comes out
+// bit for bit the same whichever kernel made it.
+#pragma once
+#include "common.h"
+
+__device__ __forceinline__ void load8_sum(const float* base, size_t index, int splits, size_t stride, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 4) {
+    float4 lo[4], hi[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float* p = base + (size_t)min(s0 + u, splits - 1) * stride + index;
+      lo[u] = *reinterpret_cast<const float4*>(p);
+      hi[u] = *reinterpret_cast<const float4*>(p + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s0 + u < splits) {
+        out[0] += lo[u].x; out[1] += lo[u].y; out[2] += lo[u].z; out[3] += lo[u].w;
+        out[4] += hi[u].x; out[5] += hi[u].y; out[6] += hi[u].z; out[7] += hi[u].w;
+      }
+  }
+}
+__device__ __forceinline__ void load8_sum(const bf16_t* base, size_t index, int, size_t, float* out) { ld8(base + index, out); }
+// The same sum (the same order of additions) with the loads of eight splits in flight at a time: for a
+// kernel in which this is a wave's only work before a barrier.
+__device__ __forceinline__ void load8_sum_wide(const float* base, size_t index, int splits, size_t stride, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float4 lo[8], hi[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float* p = base + (size_t)min(s0 + u, splits - 1) * stride + index;
+      lo[u] = *reinterpret_cast<const float4*>(p);
+      hi[u] = *reinterpret_cast<const float4*>(p + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (s0 + u < splits) {
+        out[0] += lo[u].x; out[1] += lo[u].y; out[2] += lo[u].z; out[3] += lo[u].w;
+        out[4] += hi[u].x; out[5] += hi[u].y; out[6] += hi[u].z; out[7] += hi[u].w;
+      }
+  }
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+}
+
+// A head of d elements is spread over TG = d / 8 lanes of a wave (a power of two; lane's chunk = its 8
+// elements); every lane of the group must call.  x: the elements, replaced by the result (float32, to
+// be rounded to T when stored).  weight: null = no norm.  cos_table: null = no rotation; rot: rotated
+// width, pairs (i, i + rot / 2), rot / 16 a power of two.  (qil/model.py:15-23, 42-46, 52-55)
+template <typename T>
+__device__ __forceinline__ void norm_rope8(float (&x)[8], int chunk, int TG, const float* __restrict__ weight, int d,
+                                           float eps, const float* __restrict__ cos_table,
+                                           const float* __restrict__ sin_table, int position, int rot) {
+  if (weight) {
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
+    for (int o = TG >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, QIL_WAVE);
+    const float rstd = rsqrtf(sum / (float)d + eps);
+    const float4 w0 = *reinterpret_cast<const float4*>(weight + chunk * 8);
+    const float4 w1 = *reinterpret_cast<const float4*>(weight + chunk * 8 + 4);
+    const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = round_to<T>(x[e] * rstd) * w[e];
+  }
+  if (cos_table && rot > 0) {
+    const int half_chunks = rot >> 4;                   // chunks in half of the rotated width (a power of two)
+    float other[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(x[e], half_chunks, QIL_WAVE);
+    if (chunk < 2 * half_chunks) {
+      const bool first = chunk < half_chunks;
+      const size_t at = (size_t)position * (rot >> 1) + (first ? chunk : chunk - half_chunks) * 8;
+      const float4 c0 = *reinterpret_cast<const float4*>(cos_table + at), c1 = *reinterpret_cast<const float4*>(cos_table + at + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(sin_table + at), s1 = *reinterpret_cast<const float4*>(sin_table + at + 4);
+      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = first ? x[e] * c[e] - other[e] * sn[e] : other[e] * sn[e] + x[e] * c[e];
+    }
+  }
+}

@@ -14,6 +14,7 @@
 //                                       the attention kernels load matrix-core operands for P V directly
 // Rotation pairs (i, i + rot/2), i < rot/2 (qil/model.py:42-46); elements from rot on pass unrotated.
 #include "common.h"
+#include "qk_math.h"
 
 #define QIL_MAX_HEAD_DIM 512
 
@@ -90,34 +91,6 @@ __global__ void qk_norm_rope_store_kernel(
 // reduced and the rotation partner (TG lanes... rot / 16 lanes away) is fetched with lane shuffles.
 // Takes d in {16, 32, 64, 128, 256} and a rotated width whose half is a power-of-two number of
 // 8-element chunks (rot == d always qualifies).
-__device__ __forceinline__ void load8_sum(const float* base, size_t index, int splits, size_t stride, float* out) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = 0.f;
-  for (int s0 = 0; s0 < splits; s0 += 4) {
-    float4 lo[4], hi[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float* p = base + (size_t)min(s0 + u, splits - 1) * stride + index;
-      lo[u] = *reinterpret_cast<const float4*>(p);
-      hi[u] = *reinterpret_cast<const float4*>(p + 4);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (s0 + u < splits) {
-        out[0] += lo[u].x; out[1] += lo[u].y; out[2] += lo[u].z; out[3] += lo[u].w;
-        out[4] += hi[u].x; out[5] += hi[u].y; out[6] += hi[u].z; out[7] += hi[u].w;
-      }
-  }
-}
-__device__ __forceinline__ void load8_sum(const bf16_t* base, size_t index, int, size_t, float* out) { ld8(base + index, out); }
-__device__ __forceinline__ void store8(float* p, const float* v) {
-  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
-}
-__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
-  *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
-}
-
 template <typename TD, typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_store_vec_kernel(
@@ -145,35 +118,7 @@ qk_norm_rope_store_vec_kernel(
     for (int e = 0; e < 8; ++e) st(column + (size_t)e * page_size, x[e]);
     return;
   }
-  const float* weight = is_q ? q_weight : k_weight;
-  if (weight) {
-    float sum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
-    for (int o = TG >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, QIL_WAVE);
-    const float rstd = rsqrtf(sum / (float)d + eps);
-    const float4 w0 = *reinterpret_cast<const float4*>(weight + chunk * 8);
-    const float4 w1 = *reinterpret_cast<const float4*>(weight + chunk * 8 + 4);
-    const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = round_to<T>(x[e] * rstd) * w[e];
-  }
-  if (cos_table && rot > 0) {
-    const int half_chunks = rot >> 4;                   // chunks in half of the rotated width (a power of two)
-    float other[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(x[e], half_chunks, QIL_WAVE);
-    if (chunk < 2 * half_chunks) {
-      const bool first = chunk < half_chunks;
-      const size_t at = (size_t)positions[token] * (rot >> 1) + (first ? chunk : chunk - half_chunks) * 8;
-      const float4 c0 = *reinterpret_cast<const float4*>(cos_table + at), c1 = *reinterpret_cast<const float4*>(cos_table + at + 4);
-      const float4 s0 = *reinterpret_cast<const float4*>(sin_table + at), s1 = *reinterpret_cast<const float4*>(sin_table + at + 4);
-      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = first ? x[e] * c[e] - other[e] * sn[e] : other[e] * sn[e] + x[e] * c[e];
-    }
-  }
+  norm_rope8<T>(x, chunk, TG, is_q ? q_weight : k_weight, d, eps, cos_table, sin_table, positions[token], rot);
   if (is_q) {
     store8(q_out + ((size_t)token * heads + head) * d + chunk * 8, x);
   } else {

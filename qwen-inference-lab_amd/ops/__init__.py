@@ -295,6 +295,66 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
     return q
 
 
+def _decode_parts(rows, kv_heads, max_context):
+    """(keys a part, parts) of the matrix-core decode kernel: the context is split until the chip has enough blocks."""
+    wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
+    part = min(DECODE_MAX_PART, max(DECODE_MIN_PART, -(-(-(-max_context // wanted)) // 64) * 64))
+    return part, max(1, -(-max_context // part))
+
+
+def decode_attention_takes(qkv, *, heads, kv_heads, head_dim, page_size, rotation, dtype):
+    """Whether ``decode_attention`` takes the step: a float32 ``Partials`` q/k/v product, bfloat16 caches, sizes of
+    the fused kernel."""
+    rot = rotation.rot_dim if rotation is not None else 0
+    return isinstance(qkv, Partials) and dtype == torch.bfloat16 and \
+        bool(library.load().qil_attn_decode_fused_takes(heads, kv_heads, head_dim, page_size, rot))
+
+
+def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, writes, k_cache,
+                     v_cache, page_size, block_tables, row_seq, max_context, scale, window, unmerged=False):
+    """``qk_norm_rope_store`` and ``paged_attention`` in one kernel for a step whose rows are all alone in their
+    sequences: queries, the new key and the new value are made from the partial sums ``qkv`` inside the
+    attention kernel (bit for bit what the two kernels make), the new key and value are written into the
+    pages (``writes``) and used from registers.  Returns what ``paged_attention`` returns."""
+    n = qkv.shape[0]
+    dtype = torch.bfloat16
+    _require(qkv.tensor, 'qkv', torch.float32, (qkv.splits, n, (heads + 2 * kv_heads) * head_dim))
+    _require(block_tables, 'block_tables', torch.int32)
+    _require(row_seq, 'row_seq', torch.int32, (n,))
+    _require(positions, 'positions', torch.int32, (n,))
+    _check_caches(k_cache, v_cache, dtype, kv_heads, page_size, head_dim)
+    if block_tables.ndim != 2 or block_tables.shape[1] * page_size < max_context:
+        raise ValueError('block_tables are too narrow for the longest context')
+    for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
+        if w is not None:
+            _require(w, name, torch.float32, (head_dim,))
+    cos = sin = None
+    rot = 0
+    if rotation is not None:
+        cos, sin, rot = rotation.cos, rotation.sin, rotation.rot_dim
+        _require(cos, 'cos', torch.float32)
+        _require(sin, 'sin', torch.float32, cos.shape)
+        if cos.shape[1] * 2 != rot or rot > head_dim:
+            raise ValueError('rotation tables do not fit rot_dim')
+    lib = library.load()
+    out = torch.empty((n, heads * head_dim), dtype=dtype, device=k_cache.device)
+    window_arg = int(window or 0)
+    part, parts = _decode_parts(n, kv_heads, max_context)
+    nbytes = lib.qil_attn_rows_workspace(n, heads, head_dim, parts)
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=out.device) if nbytes else None
+    _check(lib.qil_attn_decode_fused(_ptr(qkv.tensor), qkv.splits, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos),
+                                     _ptr(sin), rot, int(bool(writes)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                     block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(workspace), _ptr(out),
+                                     n, heads, kv_heads, head_dim, page_size, window_arg, float(scale), part, parts,
+                                     DECODE_WAVES, int(n * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= 64),
+                                     _stream()), 'attn_decode_fused')
+    if parts > 1:
+        result = Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg, part=part,
+                          parts=parts)
+        return result if unmerged else result.merge()
+    return out
+
+
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
                     unmerged=False):
@@ -339,9 +399,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         window_arg = int(window or 0)
         if qkv.dtype == torch.bfloat16 and lib.qil_attn_decode_takes(heads, kv_heads, head_dim, page_size):
             # matrix-core kernel; split the context until the chip has about four blocks per CU
-            wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
-            part = min(DECODE_MAX_PART, max(DECODE_MIN_PART, -(-(-(-max_context // wanted)) // 64) * 64))
-            parts = max(1, -(-max_context // part))
+            part, parts = _decode_parts(rows, kv_heads, max_context)
             nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
             workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
             _check(lib.qil_attn_decode(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),

@@ -146,6 +146,9 @@ def _declare(lib):
     lib.qil_attn_rows_workspace.restype = z
     lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
     lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_attn_decode_fused_takes.argtypes = [i, i, i, i, i]
+    lib.qil_attn_decode_fused_takes.restype = i
+    lib.qil_attn_decode_fused.argtypes = [p, i, p, p, f, p, p, i, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, p]
     lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
     lib.qil_attn_decode_takes.restype = i
     lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, p]
@@ -166,5 +169,5 @@ def _declare(lib):
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z
     for name in ('qil_embed', 'qil_add_rmsnorm', 'qil_silu_mul', 'qil_add_bias', 'qil_qk_norm_rope_store',
-                 'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_gemm_bf16_gated', 'qil_gemm_bf16_unmerged', 'qil_sample'):
+                 'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_decode_fused', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_gemm_bf16_gated', 'qil_gemm_bf16_unmerged', 'qil_sample'):
         getattr(lib, name).restype = i

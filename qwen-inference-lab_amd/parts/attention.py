@@ -56,18 +56,24 @@ class Attention(Mixer):
         p = self.p
         qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
+        norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
+                     eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
+        sizes = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim)
+        if ctx.max_query == 1 and ops.decode_attention_takes(qkv, page_size=cache.page_size, rotation=rotation,
+                                                             dtype=self.dtype, **sizes):
+            # every row alone in its sequence: norm, rotation and cache write happen inside the attention kernel
+            attended = ops.decode_attention(
+                qkv, rotation=rotation, positions=ctx.positions, writes=cache.writes, k_cache=cache.k, v_cache=cache.v,
+                page_size=cache.page_size, block_tables=cache.block_tables, row_seq=ctx.row_seq,
+                max_context=ctx.max_context, scale=self.scale, window=self.window, unmerged=True, **sizes, **norms)
+            return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)
         q = ops.qk_norm_rope_store(
-            qkv, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
-            q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
-            eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            rotation=rotation, positions=ctx.positions,
-            slots=cache.slots if cache.writes else None,
-            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype)
+            qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,
+            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype, **sizes, **norms)
         attended = ops.paged_attention(
-            q, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
-            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
+            q, k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
             max_query=ctx.max_query, max_context=ctx.max_context,
-            scale=self.scale, window=self.window, unmerged=True)
+            scale=self.scale, window=self.window, unmerged=True, **sizes)
         return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

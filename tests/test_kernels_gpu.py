@@ -351,6 +351,53 @@ def test_linear_merges_unmerged_attention(ops, lengths, window, d, heads, kv_hea
     check(biased, merged.double() @ w.double().t() + rand(out_features, seed=5).double(), dtype, scale=2)
 
 
+@pytest.mark.parametrize('lengths,page_size,d,heads,kv_heads,window,norm,rot,splits', [
+    ([2100, 1, 700, 1290, 64, 2047, 300, 33], 16, 128, 32, 8, None, True, 128, 8),     # the benchmark's sizes
+    ([1, 2, 31, 32, 33, 64, 65, 96], 8, 64, 6, 2, None, True, 64, 3),                  # every edge of a 32-key step and of a page
+    ([257, 512, 513], 32, 128, 8, 1, 100, False, 64, 1),                               # no norm, half of the head rotated, a window
+    ([40, 1000], 16, 64, 16, 1, None, True, 0, 2),                                     # 16 heads a kv head, no rotation
+    ([5000], 16, 128, 5, 5, None, True, 32, 5),                                        # one head a kv head, many parts
+])
+def test_decode_attention_fused_is_the_two_kernels(ops, lengths, page_size, d, heads, kv_heads, window, norm, rot, splits):
+    """Queries, new key and new value made inside the attention kernel from the q/k/v product's partial sums:
+    the attention result and the pages are bit for bit what qk_norm_rope_store followed by paged_attention
+    leave (the last token of every history is the step's new token)."""
+    dtype = torch.bfloat16
+    rows = len(lengths)
+    total = heads + 2 * kv_heads
+    k_cache, v_cache, table, _ = build_cache(lengths, page_size, kv_heads, d, dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    row_seq = torch.arange(rows, dtype=torch.int32).cuda()
+    slots = (table[row_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32)
+    qkv = ops.Partials(rand(splits, rows, total * d, scale=0.7, seed=21))
+    q_w = (1 + 0.1 * rand(d, seed=22)) if norm else None
+    k_w = (1 + 0.1 * rand(d, seed=23)) if norm else None
+    rotation = Rot(d, 10000.0, max(lengths), rot) if rot else None
+    sizes = dict(heads=heads, kv_heads=kv_heads, head_dim=d)
+    assert ops.decode_attention_takes(qkv, page_size=page_size, rotation=rotation, dtype=dtype, **sizes)
+    k_two, v_two = k_cache.clone(), v_cache.clone()
+    q = ops.qk_norm_rope_store(qkv, q_weight=q_w, k_weight=k_w, eps=1e-6, rotation=rotation, positions=positions,
+                               slots=slots, k_cache=k_two, v_cache=v_two, page_size=page_size, dtype=dtype, **sizes)
+    want = ops.paged_attention(q, k_cache=k_two, v_cache=v_two, page_size=page_size, block_tables=table, row_seq=row_seq,
+                               positions=positions, cu_seqlens=None, seq_starts=None, single_rows=None, n_seqs=rows,
+                               max_query=1, max_context=max(lengths), scale=d ** -0.5, window=window, **sizes)
+    k_one, v_one = k_cache.clone(), v_cache.clone()
+    got = ops.decode_attention(qkv, q_weight=q_w, k_weight=k_w, eps=1e-6, rotation=rotation, positions=positions,
+                               writes=True, k_cache=k_one, v_cache=v_one, page_size=page_size, block_tables=table,
+                               row_seq=row_seq, max_context=max(lengths), scale=d ** -0.5, window=window, **sizes)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got, want, atol=0, rtol=0)
+    same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))          # NaN-filled pages: compare the bits
+    assert same(k_one, k_two) and same(v_one, v_two), 'the pages differ'
+    # a reader of another layer's cache: nothing is written, the new token's key and value are read from the pages
+    k_read, v_read = k_two.clone(), v_two.clone()
+    read = ops.decode_attention(qkv, q_weight=q_w, k_weight=k_w, eps=1e-6, rotation=rotation, positions=positions,
+                                writes=False, k_cache=k_read, v_cache=v_read, page_size=page_size, block_tables=table,
+                                row_seq=row_seq, max_context=max(lengths), scale=d ** -0.5, window=window, **sizes)
+    torch.testing.assert_close(read, want, atol=0, rtol=0)
+    assert same(k_read, k_two) and same(v_read, v_two)
+
+
 def mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, window, scale=0.3):
     """Sequences of `lengths` cached tokens whose last `chunks[i]` positions are this step's rows."""
     k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
