@@ -156,6 +156,23 @@ __global__ void silu_mul_vec_kernel(const TD* __restrict__ gate_up, int splits, 
                                                   (g.z / (1.f + expf(-g.z))) * u.z, (g.w / (1.f + expf(-g.w))) * u.w));
 }
 
+// bfloat16 in and out, eight outputs a thread: 16-byte loads and stores (inner % 8 == 0).
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int inner,
+                                       size_t total8) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total8) return;
+  const int per_row = inner / 8;
+  const size_t n = idx / per_row;
+  const int i = (int)(idx - n * per_row) * 8;
+  float g[8], u[8], y[8];
+  ld8(gate_up + n * 2 * (size_t)inner + i, g);
+  ld8(gate_up + n * 2 * (size_t)inner + inner + i, u);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = (g[e] / (1.f + expf(-g[e]))) * u[e];
+  *reinterpret_cast<uint4*>(out + n * (size_t)inner + i) =
+      make_uint4(pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
+}
+
 // x[n, i] += bias[i]
 template <typename T>
 __global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int width, size_t total) {
@@ -219,6 +236,12 @@ int qil_silu_mul(const void* gate_up, int in_dtype, int splits, void* out, int n
   if (total == 0) return 0;
   if (splits < 1 || (in_dtype == QIL_BF16 && splits != 1)) return -1;
   const size_t stride = (size_t)n * 2 * inner;
+  if (in_dtype == QIL_BF16 && out_dtype == QIL_BF16 && inner % 8 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0)) {
+    const size_t work8 = total / 8;
+    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, dim3((unsigned)((work8 + 255) / 256)), dim3(256), 0, s,
+                       (const bf16_t*)gate_up, (bf16_t*)out, inner, work8);
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   const bool vec = inner % 4 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0);
   const size_t work = vec ? total / 4 : total;
   const unsigned blocks = (unsigned)((work + 255) / 256);
