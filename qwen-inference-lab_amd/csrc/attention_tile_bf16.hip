@@ -1,6 +1,6 @@
 // The tile kernel of attention_tile.hip for its common case, written without branches in the tile loop:
-// bfloat16, head size exactly D (64, 128 or 256), page_size % 8 == 0, a block table of a sequence that
-// fits in LDS.  Same block shape, same matrix-core formulation, same order of every sum, so a row gets
+// bfloat16, head size exactly D (64, 128 or 256), a page size that is a power of two from 8 on, a block
+// table of a sequence that fits in LDS.  Same block shape, same matrix-core formulation, same order of every sum, so a row gets
 // bit for bit the result of the general kernel (qil/model.py:59-66 is the formula of both).
 //
 // What differs is the schedule:
@@ -70,8 +70,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   const int first_tile = key_begin / BK * BK;
 
   // block-table entries of [first_tile, key_end) into LDS
-  const int first_page = ps_shift >= 0 ? first_tile >> ps_shift : first_tile / page_size;
-  const int last_page = ps_shift >= 0 ? (key_end - 1) >> ps_shift : (key_end - 1) / page_size;
+  const int first_page = first_tile >> ps_shift, last_page = (key_end - 1) >> ps_shift;
   {
     const int* table = block_tables + (size_t)seq * table_stride;
     for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS) pages[i] = table[first_page + i];
@@ -115,27 +114,31 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   uint4 k_reg[K_ITERS], v_reg[V_ITERS];
   const size_t page_stride = (size_t)kv_heads * page_size * D;
   const uint32_t k_head = (uint32_t)kvh * page_size * D, v_head = (uint32_t)kvh * D * page_size;
-  auto request = [&](int k0) {
+  auto request = [&](int k0) {                             // page_size is a power of two here: ps_shift >= 0
+    int k_page[K_ITERS], v_page[V_ITERS];
+    uint32_t k_at[K_ITERS], v_at[V_ITERS];
 #pragma unroll
-    for (int it = 0; it < K_ITERS; ++it) {
+    for (int it = 0; it < K_ITERS; ++it) {                   // all the table entries first, then all the loads
       const int idx = threadIdx.x + it * FAST_THREADS;
       const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
       const int key = min(max(k0 + kl, key_begin), key_end - 1);     // clamped onto a needed key; zeroed when published
-      const int block = ps_shift >= 0 ? key >> ps_shift : key / page_size;
-      const uint32_t offset = key - block * page_size;
-      k_reg[it] = *reinterpret_cast<const uint4*>(k_cache + (size_t)pages[block - first_page] * page_stride +
-                                                  (k_head + offset * D + dv));
+      k_page[it] = pages[(key >> ps_shift) - first_page];
+      k_at[it] = k_head + (uint32_t)(key & (page_size - 1)) * D + dv;
     }
 #pragma unroll
     for (int it = 0; it < V_ITERS; ++it) {
       const int idx = threadIdx.x + it * FAST_THREADS;
       const int grp = idx / D, dim = idx % D;
       const int key = min(max(k0 + grp * 8, key_begin & ~7), (key_end - 1) & ~7);
-      const int block = ps_shift >= 0 ? key >> ps_shift : key / page_size;
-      const uint32_t offset = key - block * page_size;
-      v_reg[it] = *reinterpret_cast<const uint4*>(v_cache + (size_t)pages[block - first_page] * page_stride +
-                                                  (v_head + (uint32_t)dim * page_size + offset));
+      v_page[it] = pages[(key >> ps_shift) - first_page];
+      v_at[it] = v_head + (uint32_t)dim * page_size + (uint32_t)(key & (page_size - 1));
     }
+#pragma unroll
+    for (int it = 0; it < K_ITERS; ++it)
+      k_reg[it] = *reinterpret_cast<const uint4*>(k_cache + (size_t)k_page[it] * page_stride + k_at[it]);
+#pragma unroll
+    for (int it = 0; it < V_ITERS; ++it)
+      v_reg[it] = *reinterpret_cast<const uint4*>(v_cache + (size_t)v_page[it] * page_stride + v_at[it]);
   };
   // Key kl of a tile (= 32 a + 8 b + 4 c + e) is row 4 b + e of score sub-tile 2 a + c: lane (r, kb) of the
   // score product then holds, in sub-tiles 2 a and 2 a + 1, the keys 32 a + 8 kb .. + 7.
@@ -326,8 +329,8 @@ static int launch_fast(const void* q, int q_stride, const void* k_cache, const v
 
 // 1 if the kernel of this file takes the sizes (bfloat16 only).
 extern "C" int qil_attn_tile_bf16_takes(int d, int page_size, int table_stride) {
-  return (d == 64 || d == 128 || d == 256) && page_size > 0 && page_size % 8 == 0 && table_stride >= 1 &&
-         table_stride <= FAST_TABLE_MAX;
+  return (d == 64 || d == 128 || d == 256) && page_size >= 8 && (page_size & (page_size - 1)) == 0 &&
+         table_stride >= 1 && table_stride <= FAST_TABLE_MAX;
 }
 
 // The arguments of qil_attn_tile (attention_tile.hip), which calls this when the sizes are taken.
