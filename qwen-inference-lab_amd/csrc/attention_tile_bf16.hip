@@ -14,6 +14,9 @@
 //    fragment while the products of the one before run;
 //  * the rows of a 16-key score tile are assigned to keys so that a lane's eight probabilities of a
 //    32-key step belong to eight consecutive keys: its V^T fragment is one 16-byte LDS read;
+//  * for D <= 128 a wave's 32 rows are ONE tile of v_mfma_f32_32x32x16_bf16, which sustains 2.1 PFLOP/s on
+//    gfx950 where the 16x16x32 shape stops near 1.3 (this kernel is bound by the matrix cores); a lane then
+//    holds 32 scores of one row, and the row's statistics need one shuffle;
 //  * for D <= 128 the LDS holds two tiles, so a tile costs one barrier: the next tile is written to
 //    the other half before this one is multiplied.
 #include <type_traits>
@@ -22,6 +25,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define FAST_THREADS 256
 #define FAST_BK 64                                         // keys per LDS tile
@@ -108,6 +112,36 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     for (int t = 0; t < DTILES; ++t) o[b][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
+  // WIDE (D <= 128): the wave's 32 rows as one 32 x 32 tile.  Lane = (row lane % 32, half lane / 32):
+  //   S^T[key, row] = K Q^T:  A = K rows (LDS), B = Q[row][dims 16 ks + 8 half ..]
+  //     -> the lane's 16 scores of a 32-key tile are the keys 16 (j / 2) + 8 half + 4 (j % 2) + e, j, e < 4
+  //        (the K rows are placed in LDS accordingly), so that scores 8 s .. 8 s + 7 are the eight
+  //        consecutive keys 16 s + 8 half .. of the tile: the B operand of
+  //   O^T[dim, row] = V^T P^T:  A = V^T[dim lane % 32][keys 16 s + 8 half ..] (one 16-byte LDS read)
+  //     -> the lane holds O[row][dims 32 t + 8 j + 4 half + e].
+  constexpr bool WIDE = RB == 2;
+  constexpr int WFRAGS = D / 16, WTILES = D / 32;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wide_row = wave_row0 + l32;
+  const bool wide_valid = wave_active && wide_row < n;
+  const int wide_pos = wide_valid ? start + wide_row : -1;
+  bf16x8 qw[WFRAGS];
+  float wide_m = -INFINITY, wide_l = 0.f;
+  f32x16 ow[WTILES];
+  if constexpr (WIDE) {
+    const bf16_t* qrow = q + (size_t)(q0 + (wide_valid ? wide_row : 0)) * q_stride + (size_t)(wave_active ? head : 0) * D;
+#pragma unroll
+    for (int ks = 0; ks < WFRAGS; ++ks) {
+      uint4 raw = make_uint4(0, 0, 0, 0);
+      if (wide_valid) raw = *reinterpret_cast<const uint4*>(qrow + ks * 16 + half * 8);
+      qw[ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+#pragma unroll
+    for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ow[t][i] = 0.f;
+  }
+
   // What this thread stages of every tile: K vector it = 16 bytes of key idx / (D / 8), V^T vector it =
   // 8 keys (one 16-byte piece of a page row) of dim idx % D.
   // Addresses: 64 bits for the page (a cache may hold more than 2^31 elements), 32 bits within it.
@@ -141,7 +175,8 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
       v_reg[it] = *reinterpret_cast<const uint4*>(v_cache + (size_t)v_page[it] * page_stride + v_at[it]);
   };
   // Key kl of a tile (= 32 a + 8 b + 4 c + e) is row 4 b + e of score sub-tile 2 a + c: lane (r, kb) of the
-  // score product then holds, in sub-tiles 2 a and 2 a + 1, the keys 32 a + 8 kb .. + 7.
+  // score product then holds, in sub-tiles 2 a and 2 a + 1, the keys 32 a + 8 kb .. + 7.  (WIDE: key
+  // 32 a + 16 s + 8 h + 4 j + e is row 16 s + 8 j + 4 h + e of 32-key tile a.)
   auto publish = [&](int k0, bf16_t* tile) {
     bf16_t* Ks = tile;
     bf16_t* Vt = tile + BK * K_ROW;
@@ -152,7 +187,8 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
       const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
       const int key = k0 + kl;
       const bool valid = inside || (key >= key_begin && key < key_end);
-      const int row = ((kl >> 5) * 2 + ((kl >> 2) & 1)) * 16 + ((kl >> 3) & 3) * 4 + (kl & 3);
+      const int row = WIDE ? (kl >> 5) * 32 + ((kl >> 4) & 1) * 16 + ((kl >> 2) & 1) * 8 + ((kl >> 3) & 1) * 4 + (kl & 3)
+                           : ((kl >> 5) * 2 + ((kl >> 2) & 1)) * 16 + ((kl >> 3) & 3) * 4 + (kl & 3);
       *reinterpret_cast<uint4*>(Ks + row * K_ROW + dv) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -252,12 +288,82 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     }
   };
 
+  auto attend_wide = [&](int k0, const bf16_t* tile, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const bf16_t* Ks = tile;
+    const bf16_t* Vt = tile + BK * K_ROW;
+    f32x16 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const bf16_t* krow = Ks + (kt * 32 + l32) * K_ROW + half * 8;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < WFRAGS; ++ks) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + ks * 16));
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qw[ks], s[kt], 0, 0, 0);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (MASKED) {
+          const int key = k0 + 32 * kt + 16 * (i >> 3) + 8 * half + (i & 7);      // j = i / 4, e = i % 4
+          const bool visible = key <= wide_pos && (window <= 0 || key > wide_pos - window);
+          s[kt][i] = visible ? s[kt][i] : -INFINITY;
+        }
+        mx = fmaxf(mx, s[kt][i]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+    const float m_new = fmaxf(wide_m, mx);
+    const float base = (m_new == -INFINITY) ? 0.f : m_new;                              // exp(-inf - 0) = 0
+    const float shift = -base * c;
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(fmaf(wide_m, c, shift));
+    float psum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[kt][i], c, shift));
+        s[kt][i] = p;
+        psum += p;
+      }
+    wide_l = wide_l * alpha + psum;
+    if (m_new != wide_m) {                       // nothing to rescale while the maximum stands
+#pragma unroll
+      for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ow[t][i] *= alpha;
+    }
+    wide_m = m_new;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const bf16x8 pb = __builtin_bit_cast(
+            bf16x8, make_uint4(pack_bf16(s[kt][8 * st], s[kt][8 * st + 1]), pack_bf16(s[kt][8 * st + 2], s[kt][8 * st + 3]),
+                               pack_bf16(s[kt][8 * st + 4], s[kt][8 * st + 5]), pack_bf16(s[kt][8 * st + 6], s[kt][8 * st + 7])));
+#pragma unroll
+        for (int t = 0; t < WTILES; ++t) {
+          const bf16x8 a = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4*>(Vt + (t * 32 + l32) * V_ROW + 32 * kt + 16 * st + 8 * half));
+          ow[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, ow[t], 0, 0, 0);
+        }
+      }
+  };
   auto attend_tile = [&](int k0, const bf16_t* tile) {
     if (wave_active && k0 <= wave_last_pos) {
       const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 16 * RB <= n &&
                                (window <= 0 || k0 > wave_last_pos - window);
-      if (all_visible) attend(k0, tile, std::false_type());
-      else attend(k0, tile, std::true_type());
+      if constexpr (WIDE) {
+        if (all_visible) attend_wide(k0, tile, std::false_type());
+        else attend_wide(k0, tile, std::true_type());
+      } else {
+        if (all_visible) attend(k0, tile, std::false_type());
+        else attend(k0, tile, std::true_type());
+      }
     }
   };
   __syncthreads();                                         // the table entries are in place
@@ -287,6 +393,19 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   }
 
   if (!wave_active) return;
+  if constexpr (WIDE) {
+    const float total = wide_l + __shfl_xor(wide_l, 32, QIL_WAVE);
+    if (!wide_valid) return;
+    const float inv = 1.f / total;
+    bf16_t* orow = out + ((size_t)(q0 + wide_row) * heads + head) * D;
+#pragma unroll
+    for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)                           // dims 32 t + 8 j + 4 half + e, e < 4: 8 bytes
+        *reinterpret_cast<uint2*>(orow + 32 * t + 8 * j + 4 * half) =
+            make_uint2(pack_bf16(ow[t][4 * j] * inv, ow[t][4 * j + 1] * inv), pack_bf16(ow[t][4 * j + 2] * inv, ow[t][4 * j + 3] * inv));
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
     float total = l[b];
