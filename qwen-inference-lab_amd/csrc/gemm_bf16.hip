@@ -16,6 +16,7 @@
 // and B[8 (l / 16) .. +7][l % 16]; it receives D[4 (l / 16) + i][l % 16], i < 4.  A and W rows are
 // both loaded with the same k assignment, so only the D layout matters for correctness.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -155,7 +156,7 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
 // fragments.  The 16-byte pieces of a row are stored at piece ^ row, so the writes (16 lanes, one
 // row) and the fragment reads (16 lanes, 16 rows, one logical piece) both spread over all banks.
 // LDS operations of one wave complete in program order, so the buffer needs no barrier.
-// Takes M <= 64, K a multiple of 128 per split, 16-byte aligned operands, no bias.
+// Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
 #define LINES_WAVES 8
 
 // A given as the unmerged partial results of split-context attention (attention_rows.hip,
@@ -213,15 +214,14 @@ __device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
                     pack_bf16(numer[4] / denom, numer[5] / denom), pack_bf16(numer[6] / denom, numer[7] / denom));
 }
 
-// MT: 16-row tiles of A (M <= 16 MT); every W fragment read from the buffer serves MT products.
-template <typename OUT, bool MERGE, int MT>
+template <typename OUT, bool MERGE>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
 gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const bf16_t* __restrict__ W,
                        OUT* __restrict__ C, int M, int N, int K, int cols_per_split) {
-  extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16 MT][cols + pad], then the waves' buffers
+  extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int a_rows = MT > 1 ? 16 * MT : M <= 8 ? 8 : 16;   // rows of A kept; the others multiply as zeros
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
   const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
   const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
   const int row_width = cols_per_split + GEMM_LDS_PAD;
@@ -260,9 +260,7 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   request(w2, 2);
   __syncthreads();
 
-  f32x4 acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   const bool a_live = r < a_rows;
   const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + kb * 8;
   auto pass = [&](const u32x4 (&stage_w)[4]) {             // registers -> buffer
@@ -275,13 +273,10 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        u32x4 a = *reinterpret_cast<const u32x4*>(a_row + t * 16 * row_width + at + s4 * 32);
-        if (MT == 1 && !a_live) a = (u32x4){0, 0, 0, 0};
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
-                                                         acc[t], 0, 0, 0);
-      }
+      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
+      if (!a_live) a = (u32x4){0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
+                                                    0, 0);
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -300,32 +295,30 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   if (left > 4) { pass(w1); multiply(stage + 4); }
   OUT* out = C + (size_t)split * M * N;
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = t * 16 + 4 * kb + i, n = n0 + r;
-      if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[t][i]);
-    }
+  for (int i = 0; i < 4; ++i) {
+    const int m = 4 * kb + i, n = n0 + r;
+    if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[i]);
+  }
 }
 
 static size_t lines_lds(int M, int K, int splits) {
-  const int rows = M <= 8 ? 8 : M <= 16 ? 16 : M <= 32 ? 32 : 64;
+  const int rows = M <= 8 ? 8 : 16;
   return ((size_t)rows * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
 }
 
 // Whether the whole-line kernel takes the product with this many splits.
 static bool lines_takes(const void* A, const void* W, const float* bias, int M, int N, int K, int splits) {
-  if (bias || M > 64 || N < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH ||
+  if (bias || M > 16 || N < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH ||
       (((uintptr_t)A | (uintptr_t)W) % 16))
     return false;
   return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
 }
 
-template <typename OUT, bool MERGE, int MT>
-static int launch_lines_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
-                              UnmergedA unmerged) {
+template <typename OUT, bool MERGE = false>
+static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
+                        UnmergedA unmerged = UnmergedA()) {
   const size_t lds = lines_lds(M, K, splits);
-  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE, MT>;
+  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE>;
   static size_t granted = 0;                              // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -337,13 +330,165 @@ static int launch_lines_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, i
   return 0;
 }
 
-template <typename OUT, bool MERGE = false>
-static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
-                        UnmergedA unmerged = UnmergedA()) {
-  if (M <= 16) return launch_lines_tiles<OUT, MERGE, 1>(A, W, C, M, N, K, splits, s, unmerged);
-  if (MERGE) return -1;                                    // the merge is made for the few rows of decode steps
-  if (M <= 32) return launch_lines_tiles<OUT, false, 2>(A, W, C, M, N, K, splits, s, unmerged);
-  return launch_lines_tiles<OUT, false, 4>(A, W, C, M, N, K, splits, s, unmerged);
+// ---------------------------------------------------------------------------------------------------
+// The whole-line product for 17 to 64 rows of A and any length of K.  A does not stay in LDS as a whole
+// slice: it passes through it one stage (128 columns) at a time, in two slots that the block's threads
+// fill in turn, from registers that are loaded three stages ahead, as W's are.  One barrier a stage: the
+// stage's slot has been written before it and the other slot may be written after it.  All waves of a
+// block are at the same stage, so the walk through K starts at a column of the block's (not the wave's) own.
+// MT: 16-row tiles of A (M <= 16 MT); every W fragment read from the buffer serves MT products.
+// Takes 16 < M <= 64, K a multiple of 128 per split with at least 3 stages, 16-byte aligned operands, no bias.
+#define CHUNK_ROW (128 + GEMM_LDS_PAD)
+
+template <typename OUT, int MT>
+__global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
+gemm_bf16_chunks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N,
+                        int K, int cols_per_split) {
+  extern __shared__ __align__(16) bf16_t lds[];            // two stages of A [16 MT][128 + pad], then the waves' buffers
+  constexpr int A_ROWS = 16 * MT, SLOT = A_ROWS * CHUNK_ROW;
+  constexpr int PIECES = A_ROWS * 16 / (LINES_WAVES * QIL_WAVE);   // 16-byte pieces of a stage of A per thread
+  static_assert(PIECES >= 1, "a stage of A has fewer pieces than the block has threads");
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
+  const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
+  bf16_t* buffer = lds + 2 * SLOT + wave * (16 * 128);
+
+  const int load_row = lane >> 4, piece = lane & 15;
+  const bf16_t* source[4];                                 // rows past N read a valid row and are never stored
+  int place[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    source[u] = W + (size_t)min(n0 + row, N - 1) * K + k_begin + piece * 8;
+    place[u] = row * 128 + ((piece ^ row) & 15) * 8;
+  }
+  // This thread's pieces of a stage of A.  Rows past M read row M - 1: their products land in rows of the
+  // result that are never stored.  (A load under a condition would make the compiler wait for every load in
+  // flight, W's too, at each stage.)
+  const bf16_t* a_source[PIECES];
+  int a_place[PIECES];
+#pragma unroll
+  for (int u = 0; u < PIECES; ++u) {
+    const int p = threadIdx.x + u * (LINES_WAVES * QIL_WAVE), row = p >> 4, pc = p & 15;
+    a_source[u] = A + (size_t)min(row, M - 1) * K + k_begin + pc * 8;
+    a_place[u] = row * CHUNK_ROW + pc * 8;
+  }
+  const int turn = blockIdx.x % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * 128; };
+  u32x4 w0[4], w1[4], w2[4], a0[PIECES], a1[PIECES], a2[PIECES];
+  auto request = [&](u32x4 (&stage_w)[4], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const u32x4*>(source[u] + at);
+  };
+  auto request_a = [&](u32x4 (&stage_a)[PIECES], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) stage_a[u] = *reinterpret_cast<const u32x4*>(a_source[u] + at);
+  };
+  auto store_a = [&](const u32x4 (&stage_a)[PIECES], int stage) {
+    bf16_t* slot = lds + (stage & 1) * SLOT;
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) *reinterpret_cast<u32x4*>(slot + a_place[u]) = stage_a[u];
+  };
+  request_a(a0, 0); request_a(a1, 1); request_a(a2, 2);     // the host sees to stages >= 3
+  request(w0, 0); request(w1, 1); request(w2, 2);
+  store_a(a0, 0);
+  if (3 < stages) request_a(a0, 3);
+  __syncthreads();
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  auto pass = [&](const u32x4 (&stage_w)[4]) {             // registers -> buffer
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = stage_w[u];
+  };
+  auto multiply = [&](int stage) {
+    const bf16_t* a_row = lds + (stage & 1) * SLOT + r * CHUNK_ROW + kb * 8;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + t * 16 * CHUNK_ROW + s4 * 32);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                         acc[t], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  // Stage s: its W goes from registers w to the buffer; registers a hold stage s + 1 of A.  `inner`: every
+  // request of the stage has a target.  (A request under a condition, even a uniform one, makes the compiler
+  // wait for all loads in flight at the next use of any of them, so the stages that need conditions are apart.)
+  auto step = [&](int s, u32x4 (&w)[4], u32x4 (&a)[PIECES], auto inner) {
+    pass(w);
+    if (decltype(inner)::value || s + 3 < stages) request(w, s + 3);
+    if (decltype(inner)::value || s + 1 < stages) store_a(a, s + 1);
+    if (decltype(inner)::value || s + 4 < stages) request_a(a, s + 4);
+    multiply(s);
+    __syncthreads();
+  };
+  int s = 0;
+  for (; s + 7 <= stages; s += 3) {
+    step(s, w0, a1, std::true_type());
+    step(s + 1, w1, a2, std::true_type());
+    step(s + 2, w2, a0, std::true_type());
+  }
+  for (; s + 3 <= stages; s += 3) {
+    step(s, w0, a1, std::false_type());
+    step(s + 1, w1, a2, std::false_type());
+    step(s + 2, w2, a0, std::false_type());
+  }
+  if (s < stages) step(s, w0, a1, std::false_type());
+  if (s + 1 < stages) step(s + 1, w1, a2, std::false_type());
+  OUT* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = t * 16 + 4 * kb + i, n = n0 + r;
+      if (m < M && n < N) store_out(out + (size_t)m * N + n, acc[t][i]);
+    }
+}
+
+static bool chunks_takes(const void* A, const void* W, const float* bias, int M, int N, int K, int splits) {
+  return !bias && M > 16 && M <= 64 && N >= 1 && splits >= 1 && K % (128 * splits) == 0 &&
+         K / (128 * splits) >= LINES_DEPTH && (((uintptr_t)A | (uintptr_t)W) % 16) == 0;
+}
+
+// K splits of that kernel when partial sums are allowed: the most (a power of two up to 8, with at least
+// three stages each) that keep the blocks within the 256 CUs; one block a CU runs them all at once, and of the
+// numbers of splits tried (1 to 8 for the products of 8B and 32B layer sizes) this one was the fastest each time.
+static int chunks_splits(int N, int K) {
+  const long tiles = (N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES);
+  int splits = 1;
+  for (int c = 2; c <= 8; c *= 2)
+    if (tiles * c <= 256 && K % (128 * c) == 0 && K / (128 * c) >= LINES_DEPTH) splits = c;
+  return splits;
+}
+
+template <typename OUT, int MT>
+static int launch_chunks_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
+  const size_t lds = ((size_t)2 * 16 * MT * CHUNK_ROW + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
+  auto kernel = gemm_bf16_chunks_kernel<OUT, MT>;
+  static size_t granted = 0;                              // per instantiation
+  if (lds > 64 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
+  return 0;
+}
+
+template <typename OUT>
+static int launch_chunks(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
+  if (M <= 32) return launch_chunks_tiles<OUT, 2>(A, W, C, M, N, K, splits, s);
+  return launch_chunks_tiles<OUT, 4>(A, W, C, M, N, K, splits, s);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -572,9 +717,17 @@ static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
 
 // How many ways the product will be split over K when partial sums are allowed.
 extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
+  if (M > 16 && M <= 64 && K % 128 == 0 && K / 128 >= LINES_DEPTH) return chunks_splits(N, K);
   int code, splits;
   plan(M, N, K, true, &code, &splits);
   return splits;
+}
+
+// 1 if a product with 17 to 64 rows has a weight-streaming kernel here (K a multiple of 128 of at least 384, no
+// bias; operands 16-byte aligned, which the call checks); products of up to 16 rows always have one.
+extern "C" int qil_gemm_bf16_streams(int M, int N, int K, int has_bias) {
+  if (M <= 16) return 1;
+  return chunks_takes(nullptr, nullptr, has_bias ? (const float*)1 : nullptr, M, N, K, 1);
 }
 
 // 1 if qil_gemm_bf16_unmerged takes these sizes (rows, output columns, heads, head size, K splits).
@@ -622,6 +775,16 @@ extern "C" int qil_gemm_bf16(const void* A, const void* W, const float* bias, vo
       QIL_RETURN_LAUNCH_STATUS();
     }
     if (code == 1) return -1;
+  }
+  if (code == 0 || code == 2) {                              // 2: force the kernel that streams A (tuning runs)
+    if (chunks_takes(A, W, bias, M, N, K, splits)) {
+      const int status = out_dtype == QIL_F32
+                             ? launch_chunks<float>((const bf16_t*)A, (const bf16_t*)W, (float*)C, M, N, K, splits, s)
+                             : launch_chunks<bf16_t>((const bf16_t*)A, (const bf16_t*)W, (bf16_t*)C, M, N, K, splits, s);
+      if (status) return status;
+      QIL_RETURN_LAUNCH_STATUS();
+    }
+    if (code == 2) return -1;
   }
   if (!code) plan(M, N, K, false, &code, &planned);
   int status;

@@ -15,11 +15,12 @@ import torch
 
 from . import library
 
-# Rows up to which a bfloat16 product runs on the weight-streaming kernel (float32 results: always).
+# Rows up to which every bfloat16 product runs on a weight-streaming kernel of this library (float32 results: always).
 STREAM_GEMM_MAX_ROWS = 16
-# ... and up to this many rows when the weight is small (elements): there the library's product is bound
-# by its launch and tiling, not by memory (measured at 24 and 32 rows: 14 us against 19 for 6144 x 4096).
-STREAM_GEMM_MORE_ROWS, STREAM_GEMM_SMALL_WEIGHT = 32, 32 * 2 ** 20
+# ... and up to this many rows where K is a multiple of 128 (at least 384) and there is no bias: the kernel that
+# passes A through LDS in stages.  Measured at 64 rows and 8B layer sizes against the GPU BLAS: 41 us against 47
+# (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).
+STREAM_GEMM_MOST_ROWS = 64
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
 # Blocks the matrix-core decode kernel aims for (256 CUs, 8 waves a block; measured best at 8 rows x 2048 keys).
@@ -30,6 +31,10 @@ DECODE_WAVES = 8
 DECODE_MIN_PART = 256
 # Most keys of a block.
 DECODE_MAX_PART = 8192
+# Rows up to which a decode step makes its queries, new keys and values inside the attention kernel: with few
+# rows that saves a launch; with many the kernel is bound by memory and the blocks' start costs more than the
+# launch (64 rows of 2048 keys: 111 us against 94 + 5).
+FUSED_DECODE_MOST_ROWS = 16
 # Launches of at most this many blocks (one a CU) let a wave load two of its steps at a time.
 DECODE_PAIRS_BLOCKS = 256
 
@@ -208,13 +213,14 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
         _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, splits, _stream()), 'gemm_f32')
         return Partials(out) if splits > 1 else out[0]
     _code(x.dtype)
-    streams = n <= STREAM_GEMM_MAX_ROWS
-    small = n <= STREAM_GEMM_MORE_ROWS and weight.numel() <= STREAM_GEMM_SMALL_WEIGHT and k % 128 == 0
-    if (streams or small) and partials and bias is None and out_dtype == x.dtype:
+    streams = n <= STREAM_GEMM_MOST_ROWS and bool(lib.qil_gemm_bf16_streams(n, o, k, bias is not None))
+    if streams and partials and bias is None and out_dtype == x.dtype:
         splits = lib.qil_gemm_bf16_splits(n, o, k)
-        out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
-        _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, 0, 0, _stream()), 'gemm_bf16')
-        return Partials(out)
+        if splits > 1 or n <= STREAM_GEMM_MAX_ROWS:
+            out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+            _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), None, _ptr(out), n, o, k, 0, splits, 0, 0, _stream()),
+                   'gemm_bf16')
+            return Partials(out)
     if out_dtype == torch.float32 or streams:
         out = torch.empty((n, o), dtype=out_dtype, device=x.device)
         _check(lib.qil_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, _code(out_dtype), 1, 0, 0,
@@ -306,7 +312,7 @@ def decode_attention_takes(qkv, *, heads, kv_heads, head_dim, page_size, rotatio
     """Whether ``decode_attention`` takes the step: a float32 ``Partials`` q/k/v product, bfloat16 caches, sizes of
     the fused kernel."""
     rot = rotation.rot_dim if rotation is not None else 0
-    return isinstance(qkv, Partials) and dtype == torch.bfloat16 and \
+    return isinstance(qkv, Partials) and qkv.shape[0] <= FUSED_DECODE_MOST_ROWS and dtype == torch.bfloat16 and \
         bool(library.load().qil_attn_decode_fused_takes(heads, kv_heads, head_dim, page_size, rot))
 
 

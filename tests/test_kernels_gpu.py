@@ -123,19 +123,44 @@ def test_linear_bfloat16(ops, m, n, k, out_dtype, bias):
 
 
 @pytest.mark.parametrize('m,n,k', [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 12288), (64, 1024, 3072), (16, 130, 52),
-                                   (3, 96, 224), (40, 200, 1030), (24, 6144, 4096), (32, 300, 1024), (17, 48, 384)])
+                                   (3, 96, 224), (40, 200, 1030), (24, 6144, 4096), (32, 300, 1024), (17, 48, 384),
+                                   (64, 6144, 4096), (48, 4096, 4096), (33, 2100, 1024), (70, 256, 512)])
 def test_linear_partial_sums(ops, m, n, k):
     """Few rows, bfloat16: the product may come back split over K; the parts add up to it."""
     x, w = rand(m, k, dtype=torch.bfloat16), rand(n, k, dtype=torch.bfloat16, seed=1, scale=k ** -0.5)
     got = ops.linear(x, w, None, partials=True)
-    if not isinstance(got, ops.Partials):                  # many rows: the library's product, in bfloat16
-        assert m > ops.STREAM_GEMM_MORE_ROWS or (m > ops.STREAM_GEMM_MAX_ROWS and k % 128)
+    if not isinstance(got, ops.Partials):                  # many rows, or a K that is not split: one bfloat16 result
+        whole = k % 128 or k < 384 or ops.library.load().qil_gemm_bf16_splits(m, n, k) == 1
+        assert m > ops.STREAM_GEMM_MOST_ROWS or (m > ops.STREAM_GEMM_MAX_ROWS and whole)
         check(got, x.double() @ w.double().t(), torch.bfloat16, scale=2)
         return
     assert isinstance(got, ops.Partials) and got.shape == (m, n)
     check(got.sum(), x.double() @ w.double().t(), torch.float32, scale=8)
     if k >= 4096 and n <= 8192:
         assert got.splits > 1, 'a product with few columns and a long K should be split'
+
+
+@pytest.mark.parametrize('k', [384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 2432])
+@pytest.mark.parametrize('m', [17, 32, 33, 64])
+def test_linear_17_to_64_rows(ops, m, k):
+    """The kernel that passes A through LDS in stages, at every number of stages from 3 on (the first and the
+    last stages run apart from the inner ones), at both numbers of row tiles, with rows of W past the end
+    of a wave's and of a block's sixteen, whole and split over K."""
+    n = 130 if k != 1024 else 2100
+    x, w = rand(m, k, dtype=torch.bfloat16), rand(n, k, dtype=torch.bfloat16, seed=1, scale=k ** -0.5)
+    want = x.double() @ w.double().t()
+    assert ops.library.load().qil_gemm_bf16_streams(m, n, k, 0) == 1
+    check(ops.linear(x, w, None, out_dtype=torch.float32), want, torch.float32, scale=8)
+    check(ops.linear(x, w, None), want, torch.bfloat16, scale=2)
+    got = ops.linear(x, w, None, partials=True)
+    if isinstance(got, ops.Partials):
+        assert got.splits > 1
+        check(got.sum(), want, torch.float32, scale=8)
+    else:
+        check(got, want, torch.bfloat16, scale=2)
+    # a row's result does not depend on the rows beside it
+    alone = ops.linear(x[m - 17:].contiguous(), w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(alone, ops.linear(x, w, None, out_dtype=torch.float32)[m - 17:], atol=0, rtol=0)
 
 
 def test_linear_rows_do_not_depend_on_the_batch(ops):
