@@ -98,13 +98,35 @@ qk_norm_rope_store_vec_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size,
-    float eps, int tg_log2) {
+    float eps, int tg_log2, unsigned v_first_block) {
   const int total_heads = heads + 2 * kv_heads;
   const int TG = 1 << tg_log2;
+  if (blockIdx.x >= v_first_block) {
+    // v apart (TG >= 4): a wave takes 16 tokens x 4 chunks of one head, so that a store instruction (one
+    // element of every lane's chunk) fills 32 contiguous bytes per chunk when the tokens follow each other
+    // in a page, instead of touching 64 lines with 2 bytes each.  v: copy, transposed within the page.
+    const int lane = threadIdx.x & (QIL_WAVE - 1);
+    const size_t wave = (size_t)(blockIdx.x - v_first_block) * (blockDim.x / QIL_WAVE) + threadIdx.x / QIL_WAVE;
+    const int quads = TG >> 2;
+    const int quad = (int)(wave % quads), kvh = (int)(wave / quads % kv_heads);
+    const size_t group = wave / quads / kv_heads;
+    const size_t token = group * 16 + (lane >> 2);
+    const int chunk = quad * 4 + (lane & 3);
+    if (token >= (size_t)n) return;
+    float x[8];
+    load8_sum(qkv, (token * total_heads + heads + kv_heads + kvh) * d + chunk * 8, splits, split_stride, x);
+    const int slot = slots[token];
+    const size_t page = slot / page_size, offset = slot % page_size;
+    T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + chunk * 8) * page_size + offset;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) st(column + (size_t)e * page_size, x[e]);
+    return;
+  }
+  const int pair_heads = v_first_block != 0xffffffffu ? heads + kv_heads : total_heads;   // v apart: q and k only here
   const int pair = (int)((blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> tg_log2);    // (token, head) pair
   const int chunk = threadIdx.x & (TG - 1);
-  if (pair >= n * total_heads) return;                  // whole lane groups leave together
-  const int token = pair / total_heads, head = pair - token * total_heads;
+  if (pair >= n * pair_heads) return;                   // whole lane groups leave together
+  const int token = pair / pair_heads, head = pair - token * pair_heads;
   const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
   if (!is_q && slots == nullptr) return;
   float x[8];
@@ -148,12 +170,17 @@ extern "C" int qil_qk_norm_rope_store(
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)q_weight | (uintptr_t)k_weight |
                          (uintptr_t)cos_table | (uintptr_t)sin_table) % 16) == 0;
   if (tg_log2 > 0 && rot_fits && aligned) {
-    const size_t lanes = (size_t)n * (heads + 2 * kv_heads) << tg_log2;
-    const unsigned blocks = (unsigned)((lanes + 255) / 256);
+    // v in blocks of its own behind the others when a head has at least four chunks and there is a cache to write
+    const bool v_apart = tg_log2 >= 2 && slots != nullptr;
+    const size_t lanes = (size_t)n * (v_apart ? heads + kv_heads : heads + 2 * kv_heads) << tg_log2;
+    const unsigned pair_blocks = (unsigned)((lanes + 255) / 256);
+    const size_t v_waves = v_apart ? (size_t)((n + 15) / 16) * kv_heads * ((size_t)1 << (tg_log2 - 2)) : 0;
+    const unsigned v_first_block = v_apart ? pair_blocks : 0xffffffffu;
+    const unsigned blocks = pair_blocks + (unsigned)((v_waves + 3) / 4);
 #define QIL_QKV_CASE(TD, T)                                                                                           \
   hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)qkv, splits,    \
                      stride, (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache,       \
-                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2)
+                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block)
     if (dtype == QIL_F32) QIL_QKV_CASE(float, float);
     else if (in_dtype == QIL_F32) QIL_QKV_CASE(float, bf16_t);
     else QIL_QKV_CASE(bf16_t, bf16_t);
