@@ -525,12 +525,23 @@ REAL = {
                intermediate_size=12288, num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8,
                head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
                attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=None),
+    # a width and an inner width that are no multiple of 1024 (20 and 76 stages of 128 columns)
+    '4B': dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=151936, hidden_size=2560,
+               intermediate_size=9728, num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8,
+               head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
+               attention_bias=False, tie_word_embeddings=True, hidden_act='silu', eos_token_id=None),
+    # five query heads to a key/value head
+    '14B': dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=151936, hidden_size=5120,
+                intermediate_size=17408, num_hidden_layers=1, num_attention_heads=40, num_key_value_heads=8,
+                head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=None),
 }
 
 
-@pytest.mark.parametrize('name,dtype', [('0.6B', torch.float32), ('0.6B', torch.bfloat16), ('8B', torch.bfloat16)])
+@pytest.mark.parametrize('name,dtype', [('0.6B', torch.float32), ('0.6B', torch.bfloat16), ('8B', torch.bfloat16),
+                                        ('4B', torch.bfloat16), ('14B', torch.bfloat16)])
 def test_layers_of_real_size(tmp_path, name, dtype):
-    """Few layers at the sizes of Qwen3-0.6B / 8B (head size 128, vocabulary 151,936): a mixed, chunked
+    """Few layers at the sizes of Qwen3-0.6B / 4B / 8B / 14B (head size 128, vocabulary 151,936): a mixed, chunked
     replay of three requests against the plain implementation, and a greedy step through the sampler."""
     from qil_amd.engine import ModelRunner, StepEntry
     from qil_amd.sampling import Sampler, SamplingParams
