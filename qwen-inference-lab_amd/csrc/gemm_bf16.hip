@@ -1,5 +1,8 @@
 // bfloat16 matrix product on the matrix cores for few rows (decode, selected logit rows):
 //   C[M, N] = A[M, K] W[N, K]^T (+ bias[N]),  float32 accumulation.
+// Four kernels, all bound by reading W once: `stream` (this comment; any shape, bias, unaligned operands),
+// `lines` (up to 16 rows, W in whole cache lines, optional merge of attention parts into A), `chunks`
+// (17 to 64 rows, A through LDS in stages) and `gated` (gate and up products with SiLU in the epilogue).
 // Both operands have K contiguous (qil/model.py:32-40).  The product is bound by streaming W once
 // from HBM; A is small and would be re-read from L2 by every block, so the work is cut into wide,
 // short pieces: a block owns 128 * NT rows of W (8 waves, each 16 * NT rows) and ONE of `splits`
