@@ -81,7 +81,8 @@ def main():
         args.layers = sizes['num_hidden_layers']
     config = dict(sizes, num_hidden_layers=args.layers)
     longest = args.history + args.warmup + args.steps + 2 * max([args.batch] + [int(b) for b in args.points.split(',') if b]) + 8
-    if longest > config['max_position_embeddings']:             # --history beyond the size set's context
+    longest = max(longest, args.prefill_tokens)
+    if longest > config['max_position_embeddings']:             # --history or --prefill-tokens beyond the size set's context
         config['max_position_embeddings'] = longest
     dtype = getattr(torch, args.dtype)
     element = 2 if args.dtype == 'bfloat16' else 4
