@@ -316,6 +316,11 @@ ATT_TOL = {torch.float32: dict(atol=2e-6, rtol=2e-5), torch.bfloat16: dict(atol=
     ([3, 257], 7, 256, 8, 1),
     ([300, 2], 4, 48, 5, 1),
     ([700], 16, 128, 64, 8),
+    ([33, 200], 16, 80, 8, 2),                                  # head sizes in steps of 16
+    ([129], 8, 96, 6, 3),
+    ([64, 7], 16, 112, 4, 1),
+    ([40, 300], 16, 32, 4, 2),
+    ([19, 130], 8, 160, 4, 2),
 ])
 def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, kv_heads):
     k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
@@ -468,6 +473,11 @@ def test_prompt_rows_and_window(ops, dtype, window):
     ([66, 40, 20], [35, 40, 2], 8, 16, 4, 4),                   # g = 1, head size 16
     ([513], [513], 16, 64, 4, 2),                               # g = 2
     ([2048], [2048], 16, 128, 8, 2),
+    ([150, 40], [150, 13], 16, 80, 8, 2),                       # head sizes in steps of 16
+    ([200], [77], 8, 96, 6, 3),
+    ([90, 30], [45, 30], 16, 112, 4, 1),
+    ([100], [100], 16, 32, 4, 2),
+    ([70, 20], [70, 9], 8, 160, 4, 2),
 ])
 def test_prompt_portions_against_float64(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads):
     mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, None, scale=d ** -0.5)
