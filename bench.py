@@ -65,8 +65,9 @@ def main():
     parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
     parser.add_argument('--points', default='1,64', help='other decode batch sizes to report, comma separated')
     parser.add_argument('--prefill-tokens', type=int, default=2048)
-    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill'],
-                        help='measure only one phase (for profiling); the JSON line then lacks the other')
+    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill', 'e2e'],
+                        help='measure only one phase (for profiling); the JSON line then lacks the other.  e2e: the '
+                             'reference\'s own workloads (output tokens over the wall time of whole requests)')
     args = parser.parse_args()
     if args.gpus != 1:
         print(f'bench.py measures one GPU: this engine runs on a single MI355X (asked for {args.gpus})')
@@ -142,6 +143,29 @@ def main():
     def note(text):
         print(f'[bench] {text}', file=sys.stderr, flush=True)
 
+    if args.phase == 'e2e':
+        # The reference's published workloads (docs/prefill-gpu-validation-2026-09-20.md:26-31, README.md:38-41):
+        # 1 or 4 requests with prompts of 128 / 512 / 2048 tokens, 32 output tokens each, greedy, 16-token pages,
+        # token budget 512, portions of 128, 4 active; one warm-up, the median of five runs; output tokens over
+        # the wall time of the whole batch (prefill and decode).
+        table = {}
+        for length in (128, 512, 2048):
+            for count in (1, 4):
+                engine = Engine(model, num_pages=640 if length == 2048 else 256, page_size=16, token_budget=512,
+                                prefill_chunk=128, max_active=4)
+                times = []
+                for attempt in range(6):
+                    prompts = [prompt(length) for _ in range(count)]
+                    torch.cuda.synchronize()
+                    started = time.perf_counter()
+                    results = engine.generate(prompts, max_new_tokens=32, ignore_eos=True)
+                    times.append(time.perf_counter() - started)
+                    assert all(len(r['token_ids']) == 32 for r in results)
+                engine.close()
+                table[f'{length}x{count}'] = round(32 * count / statistics.median(times[1:]), 1)
+        print(json.dumps({'e2e_output_tokens_per_s': table, 'sizes': NAMES[args.sizes], 'layers': args.layers,
+                          'dtype': args.dtype}))
+        return 0
     if args.phase == 'prefill':
         prefill_s = prefill_run(args.prefill_tokens)
         print(json.dumps({'prefill_ms': round(prefill_s * 1e3, 3), 'tokens': args.prefill_tokens, 'layers': args.layers}))

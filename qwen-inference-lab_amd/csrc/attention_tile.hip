@@ -50,8 +50,10 @@ __device__ __forceinline__ float scaled_exp(float x, float base, float scale, fl
 
 // RB: 16-row tiles per wave.  A K or V^T fragment read from LDS serves RB products, which is what
 // keeps the kernel from being bound by LDS reads.
+// (float32 with head sizes above 64 needs more than 256 registers: one block a CU there, so that what does not
+// fit goes to the other half of the register file and not to memory)
 template <typename T, int DMAX, int RB>
-__global__ void __launch_bounds__(TILE_THREADS, 2)
+__global__ void __launch_bounds__(TILE_THREADS, (sizeof(T) == 4 && DMAX > 64) ? 1 : 2)
 attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                  const int* __restrict__ block_tables, int table_stride, const int* __restrict__ cu_seqlens,
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
@@ -124,9 +126,11 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
         qb[b][ks] = __builtin_bit_cast(bf16x8, raw);
       }
     } else {
+      // step 4 j + i of a row's product takes dim 16 j + 4 kb + i from this lane: four steps' K values are one
+      // 16-byte LDS read (any assignment of dims to steps will do, as long as K and Q share it)
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks) {
-        const int dim = ks * 4 + kb;
+        const int dim = (ks >> 2) * 16 + 4 * kb + (ks & 3);
         qf[b][ks] = (row_valid[b] && dim < d) ? qrow[dim] : 0.f;
       }
     }
@@ -303,11 +307,17 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
         }
       } else {
 #pragma unroll
-        for (int ks = 0; ks < QFRAGS; ++ks)
-          if (ks * 4 < d) {
-            const float a = krow[ks * 4 + kb];
+        for (int j = 0; j < QFRAGS / 4; ++j)
+          if (j * 16 < d) {
+            // dims 16 j + 4 kb + i; past d (a head size that is no multiple of 16) the row's padding or the next
+            // row is read, finite values that meet zeros of Q
+            const f32x4 a = *reinterpret_cast<const f32x4*>(krow + j * 16 + 4 * kb);
 #pragma unroll
-            for (int b = 0; b < RB; ++b) s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, qf[b][ks], s[b][jt], 0, 0, 0);
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+              for (int b = 0; b < RB; ++b)
+                s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], qf[b][4 * j + i], s[b][jt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);              // reads of all 32 steps at once would spill
           }
       }
     }
@@ -394,14 +404,16 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
       for (int jt = 0; jt < SUB; ++jt) {
         if (k0 + jt * 16 > wave_last_pos) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int t = 0; t < DTILES; ++t)
+          if (t < dt) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(Vt + (t * 16 + r) * v_row + jt * 16 + 4 * kb);
 #pragma unroll
-          for (int t = 0; t < DTILES; ++t)
-            if (t < dt) {
-              const float a = Vt[(t * 16 + r) * v_row + jt * 16 + 4 * kb + i];
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-              for (int b = 0; b < RB; ++b) o[b][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, s[b][jt][i], o[b][t], 0, 0, 0);
-            }
+              for (int b = 0; b < RB; ++b)
+                o[b][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], s[b][jt][i], o[b][t], 0, 0, 0);
+            if (t & 1) __builtin_amdgcn_sched_barrier(0);   // reads of all dim tiles at once would spill
+          }
       }
     }
   }
