@@ -514,6 +514,56 @@ def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
         torch.testing.assert_close(pieces[name].double().cpu(), wanted[name], atol=2e-5, rtol=2e-4)
 
 
+def test_serving_loop_under_random_arrivals(model_folder):
+    """A few hundred requests of mixed lengths arrive at random, some are cancelled, some sample with a
+    temperature, with so few pages that many wait: every request ends, every page comes back, and the greedy
+    ones that completed produced the plain implementation's tokens (float32)."""
+    import random
+    from qil_amd import Engine, Qwen3
+    config = plain.TINY_B
+    folder, weights = model_folder(config, 3)
+    model = Qwen3.from_directory(folder, device='cuda', dtype=torch.float32)
+    engine = Engine(model, num_pages=300, page_size=4, token_budget=96, prefill_chunk=32, max_active=24)
+    rng, generator = random.Random(7), torch.Generator().manual_seed(1)
+    total, submitted, steps = 200, 0, 0
+    asked, pending, done = {}, set(), {}
+    while len(done) < total:
+        while submitted < total and rng.random() < 0.6:
+            new = rng.choice([1, 2, 7, 30, 64])
+            length = min(rng.choice([1, 2, 3, 5, 17, 40, 90, 200]), config['max_position_embeddings'] - new)
+            prompt = torch.randint(0, config['vocab_size'], (length,), generator=generator).tolist()
+            temperature = rng.choice([0.0, 0.0, 0.8])
+            request = engine.submit(prompt, max_new_tokens=new, ignore_eos=rng.random() < 0.5, temperature=temperature,
+                                    seed=submitted)
+            asked[request] = (prompt, new, temperature)
+            pending.add(request)
+            submitted += 1
+        if pending and rng.random() < 0.02:
+            engine.cancel(rng.choice(sorted(pending)))
+        engine.step()
+        steps += 1
+        assert steps < 5000, 'the loop does not end'
+        for request in sorted(pending):
+            result = engine.result(request)
+            if result['state'] in ('completed', 'cancelled', 'failed'):
+                done[request] = result
+                pending.discard(request)
+        if steps % 100 == 0:
+            engine.cache.check()
+    engine.cache.check()
+    assert engine.idle and engine.cache.free_pages == [300]
+    assert all(r['state'] in ('completed', 'cancelled') for r in done.values())
+    checked = 0
+    for request, result in sorted(done.items())[:60]:
+        prompt, new, temperature = asked[request]
+        if temperature == 0.0 and result['state'] == 'completed':
+            got = result['token_ids']
+            assert plain.greedy(prompt, new, weights, config)[:len(got)] == got
+            checked += 1
+    assert checked > 10
+    engine.close()
+
+
 # ------------------------------------------------------------------------------- real layer sizes
 
 REAL = {
