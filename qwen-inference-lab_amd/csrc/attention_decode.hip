@@ -62,6 +62,8 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
                    float* __restrict__ part_l, bf16_t* __restrict__ out, int heads, int kv_heads, int d,
                    int page_size, int window, float scale, int P, int parts) {
   constexpr int QFRAGS = DMAX / 32, DTILES = DMAX / 16;
+  if (FUSED) d = DMAX;                                      // what the host has checked, known to the compiler: no
+                                                            // condition on the head size stays in the loops
   extern __shared__ float lds[];
   const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
   const int row = row_index ? row_index[slot_row] : slot_row;

@@ -50,10 +50,13 @@ __device__ __forceinline__ float scaled_exp(float x, float base, float scale, fl
 
 // RB: 16-row tiles per wave.  A K or V^T fragment read from LDS serves RB products, which is what
 // keeps the kernel from being bound by LDS reads.
-// (float32 with head sizes above 64 needs more than 256 registers: one block a CU there, so that what does not
-// fit goes to the other half of the register file and not to memory)
-template <typename T, int DMAX, int RB>
-__global__ void __launch_bounds__(TILE_THREADS, (sizeof(T) == 4 && DMAX > 64) ? 1 : 2)
+// (float32 with head sizes above 64 needs more than 256 registers unless the head size is known at compile time
+// and at most 128: one block a CU there, so that what does not fit goes to the other half of the register file and
+// not to memory)
+// WHOLE: d == DMAX, known when the kernel is compiled: no condition on the head size remains in the loops over
+// dim tiles (with such conditions the float32 kernel spent most of its time copying accumulators between registers).
+template <typename T, int DMAX, int RB, bool WHOLE>
+__global__ void __launch_bounds__(TILE_THREADS, (sizeof(T) == 4 && DMAX > 64 && (!WHOLE || DMAX > 128)) ? 1 : 2)
 attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                  const int* __restrict__ block_tables, int table_stride, const int* __restrict__ cu_seqlens,
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
@@ -93,7 +96,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
   const int key_end = pos_first + rows_in_block;                       // last position + 1
   const int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
 
-  const int dt = (d + 15) / 16;                        // dim tiles in use
+  const int dt = WHOLE ? DMAX / 16 : (d + 15) / 16;    // dim tiles in use
   const int k_row = (BF16 ? (d + 31) / 32 * 32 : dt * 16) + PAD;       // elements per K row in LDS (staging
                                                                        // writes whole dim tiles)
   const int v_row = BK + PAD;                                          // elements per V^T row in LDS
@@ -131,7 +134,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
 #pragma unroll
       for (int ks = 0; ks < QFRAGS; ++ks) {
         const int dim = (ks >> 2) * 16 + 4 * kb + (ks & 3);
-        qf[b][ks] = (row_valid[b] && dim < d) ? qrow[dim] : 0.f;
+        qf[b][ks] = (row_valid[b] && (WHOLE || dim < d)) ? qrow[dim] : 0.f;
       }
     }
   }
@@ -299,7 +302,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
       if constexpr (BF16) {
 #pragma unroll
         for (int ks = 0; ks < QFRAGS; ++ks) {
-          if (ks * 32 < d) {
+          if (WHOLE || ks * 32 < d) {
             const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow + ks * 32 + kb * 8));
 #pragma unroll
             for (int b = 0; b < RB; ++b) s[b][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[b][ks], s[b][jt], 0, 0, 0);
@@ -308,7 +311,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
       } else {
 #pragma unroll
         for (int j = 0; j < QFRAGS / 4; ++j)
-          if (j * 16 < d) {
+          if (WHOLE || j * 16 < d) {
             // dims 16 j + 4 kb + i; past d (a head size that is no multiple of 16) the row's padding or the next
             // row is read, finite values that meet zeros of Q
             const f32x4 a = *reinterpret_cast<const f32x4*>(krow + j * 16 + 4 * kb);
@@ -389,7 +392,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
         }
 #pragma unroll
         for (int t = 0; t < DTILES; ++t) {
-          if (t < dt) {
+          if (WHOLE || t < dt) {
             const T* vrow = Vt + (t * 16 + r) * v_row + st * 32 + 4 * kb;
             const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
             const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
@@ -405,7 +408,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
         if (k0 + jt * 16 > wave_last_pos) continue;
 #pragma unroll
         for (int t = 0; t < DTILES; ++t)
-          if (t < dt) {
+          if (WHOLE || t < dt) {
             const f32x4 a = *reinterpret_cast<const f32x4*>(Vt + (t * 16 + r) * v_row + jt * 16 + 4 * kb);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -432,7 +435,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int dim = t * 16 + 4 * kb + i;
-        if (dim < d) st(orow + dim, o[b][t][i] * inv);
+        if (WHOLE || dim < d) st(orow + dim, o[b][t][i] * inv);
       }
   }
 }
@@ -448,12 +451,13 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
   const bool bf16 = sizeof(T) == 2;
   const int k_row = (bf16 ? (d + 31) / 32 * 32 : (d + 15) / 16 * 16) + TT::PAD, v_row = TT::BK + TT::PAD;
   const size_t lds = ((size_t)TT::BK * k_row + (size_t)((d + 15) / 16 * 16) * v_row) * sizeof(T);
-  auto kernel = attn_tile_kernel<T, DMAX, RB>;
-  static size_t granted = 0;                     // per instantiation
-  if (lds > 64 * 1024 && lds > granted) {
+  const bool whole = !bf16 && d == DMAX;                 // (the common bfloat16 sizes have a kernel of their own)
+  auto kernel = whole ? attn_tile_kernel<T, DMAX, RB, sizeof(T) == 4> : attn_tile_kernel<T, DMAX, RB, false>;
+  static size_t granted[2] = {0, 0};                     // per instantiation
+  if (lds > 64 * 1024 && lds > granted[whole]) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    granted = lds;
+    granted[whole] = lds;
   }
   dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks);
   int ps_shift = -1;                                      // log2 of a power-of-two page size
