@@ -53,7 +53,8 @@ __device__ __forceinline__ uint4 shuffle4(uint4 v, int source) {
                     __shfl(v.w, source, QIL_WAVE));
 }
 
-template <int DMAX, bool PAIRS, bool FUSED>
+// WHOLE: d == DMAX (always so when FUSED).
+template <int DMAX, bool PAIRS, bool FUSED, bool WHOLE = FUSED>
 __global__ void __launch_bounds__(DEC_MAX_WAVES * QIL_WAVE)
 attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
@@ -62,7 +63,7 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
                    float* __restrict__ part_l, bf16_t* __restrict__ out, int heads, int kv_heads, int d,
                    int page_size, int window, float scale, int P, int parts) {
   constexpr int QFRAGS = DMAX / 32, DTILES = DMAX / 16;
-  if (FUSED) d = DMAX;                                      // what the host has checked, known to the compiler: no
+  if (WHOLE) d = DMAX;                                      // what the host has checked, known to the compiler: no
                                                             // condition on the head size stays in the loops
   extern __shared__ float lds[];
   const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
@@ -373,13 +374,21 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                      table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
                      page_size, window, scale, P, parts)
+#define QIL_DEC_WHOLE(DMAX, PAIRS)                                                                                  \
+  hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, false, true>), grid, dim3(waves * QIL_WAVE), lds, s, none,     \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
+                     table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
+                     page_size, window, scale, P, parts)
 #define QIL_DEC_CASE(DMAX)                                                                                          \
-  if (pairs) QIL_DEC_LAUNCH(DMAX, true, false, none);                                                               \
+  if (d == DMAX && pairs) QIL_DEC_WHOLE(DMAX, true);                                                                \
+  else if (d == DMAX) QIL_DEC_WHOLE(DMAX, false);                                                                   \
+  else if (pairs) QIL_DEC_LAUNCH(DMAX, true, false, none);                                                          \
   else QIL_DEC_LAUNCH(DMAX, false, false, none)
   if (d <= 64) QIL_DEC_CASE(64);
   else if (d <= 128) QIL_DEC_CASE(128);
   else QIL_DEC_CASE(256);
 #undef QIL_DEC_CASE
+#undef QIL_DEC_WHOLE
   QIL_RETURN_LAUNCH_STATUS();
 }
 
