@@ -224,7 +224,7 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept (8 or 16: a power of two)
   const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
   const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
   const int row_width = cols_per_split + GEMM_LDS_PAD;
@@ -264,8 +264,8 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
   __syncthreads();
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  const bool a_live = r < a_rows;
-  const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + kb * 8;
+  // lanes past the kept rows read the rows again: their products are rows of D that are never stored
+  const bf16_t* a_row = a_lds + (r & (a_rows - 1)) * row_width + kb * 8;
   auto pass = [&](const u32x4 (&stage_w)[4]) {             // registers -> buffer
 #pragma unroll
     for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = stage_w[u];
@@ -276,8 +276,7 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
-      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
-      if (!a_live) a = (u32x4){0, 0, 0, 0};
+      const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
                                                     0, 0);
     }
@@ -512,7 +511,7 @@ __global__ void __launch_bounds__(GATED_MAX_WAVES * QIL_WAVE)
 gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ out, int M,
                        int inner, int K, int ksplit) {
   extern __shared__ __align__(16) bf16_t lds[];            // A [8 or 16][K + pad], then a 4 KB buffer per wave
-  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept; the others multiply as zeros
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept (8 or 16: a power of two)
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
   const int pair = wave / ksplit, part = wave - pair * ksplit;
@@ -559,8 +558,8 @@ gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
   __syncthreads();
 
   f32x4 gate = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
-  const bool a_live = r < a_rows;
-  const bf16_t* a_row = a_lds + (a_live ? r : 0) * row_width + k_begin + kb * 8;
+  // lanes past the kept rows read the rows again: their products are rows of D that are never stored
+  const bf16_t* a_row = a_lds + (r & (a_rows - 1)) * row_width + k_begin + kb * 8;
   auto pass = [&](const u32x4 (&w)[4]) {                   // registers -> buffer
 #pragma unroll
     for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = w[u];
@@ -571,8 +570,7 @@ gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
-      u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
-      if (!a_live) a = (u32x4){0, 0, 0, 0};
+      const u32x4 a = *reinterpret_cast<const u32x4*>(a_row + at + s4 * 32);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
                                                     0, 0);
     }
