@@ -12,6 +12,21 @@ __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
 }
 
+// The same for rows of bfloat16 whose width is a multiple of 8, 16-byte aligned: one thread, eight elements.
+__global__ void embed_bf16x8_kernel(const int* __restrict__ tokens, const bf16_t* __restrict__ table,
+                                    float* __restrict__ stream, int width) {
+  const int n = blockIdx.x;
+  const bf16_t* row = table + (size_t)tokens[n] * width;
+  float* out = stream + (size_t)n * width;
+  for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(row + i);
+    *reinterpret_cast<float4*>(out + i) = make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                                                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+    *reinterpret_cast<float4*>(out + i + 4) = make_float4(__uint_as_float(raw.z << 16), __uint_as_float(raw.z & 0xffff0000u),
+                                                          __uint_as_float(raw.w << 16), __uint_as_float(raw.w & 0xffff0000u));
+  }
+}
+
 __device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ float4 load4(const bf16_t* p) {
   const uint2 raw = *reinterpret_cast<const uint2*>(p);
@@ -188,6 +203,9 @@ int qil_embed(const int* tokens, const void* table, float* stream, int n, int wi
   const int threads = width >= 1024 ? 256 : 64;
   if (dtype == QIL_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, s, tokens, (const float*)table, stream, width);
+  else if (width % 8 == 0 && (((uintptr_t)table | (uintptr_t)stream) % 16) == 0)
+    hipLaunchKernelGGL(embed_bf16x8_kernel, dim3(n), dim3(width >= 2048 ? 256 : 64), 0, s, tokens, (const bf16_t*)table,
+                       stream, width);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, tokens, (const bf16_t*)table, stream, width);
   QIL_RETURN_LAUNCH_STATUS();
