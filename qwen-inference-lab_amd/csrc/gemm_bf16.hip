@@ -624,9 +624,11 @@ static size_t gated_lds(int M, int K, int waves) {
 static bool gated_plan(const void* A, const void* W, int M, int inner, int K, int* pairs, int* ksplit) {
   if (M < 1 || M > 16 || inner < 16 || inner % 16 || K % 128 || (((uintptr_t)A | (uintptr_t)W) % 16))
     return false;
+  // Most waves a pair that still leave 16 stages each; while the waves of all pairs are fewer than the machine
+  // holds (256 CUs x 8), 2 stages each will do: a small product is bound by the loads in flight, not by LDS sums.
   int ks = 0;
-  for (int c = 8; c >= 1 && !ks; c /= 2)                   // most waves that still leave 16 stages each; else 2 stages
-    if (K % (128 * c) == 0 && K / (128 * c) >= (c == 1 ? 2 : 16)) ks = c;
+  for (int c = 8; c >= 1 && !ks; c /= 2)
+    if (K % (128 * c) == 0 && K / (128 * c) >= (c == 1 || (long)(inner / 16) * c <= 2048 ? 2 : 16)) ks = c;
   if (!ks) return false;
   // Pairs a block: what a CU has to do in all (its blocks one after the other, as many at a time as LDS and
   // the 12 wave slots allow) over how well its waves keep memory busy (8 or more do).  Ties go to more pairs.
@@ -711,6 +713,14 @@ static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
     if (sp > most) sp = most;
     while (sp > 1 && steps / sp < 8) --sp;
     if (sp < 1) sp = 1;
+    // up to 16 rows: the most splits not above that which the whole-line kernel takes (whole stages of 128
+    // columns, at least LINES_DEPTH of them), if there is such a number
+    if (M <= 16 && K % 128 == 0) {
+      int fit = 0;
+      for (int c = sp; c >= 1 && !fit; --c)
+        if (K % (128 * c) == 0 && K / (128 * c) >= LINES_DEPTH) fit = c;
+      if (fit) sp = fit;
+    }
   }
   *code = mt * 100 + 10 + 4;
   *splits = sp;
