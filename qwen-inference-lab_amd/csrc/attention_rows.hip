@@ -65,22 +65,32 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[h][e] = 0.f;
     }
-    for (int t = wave * TPW + slot; t < count; t += ATT_WAVES * TPW) {
-      const int j = begin + t;
-      const size_t page = table[j / page_size];
-      const size_t base = ((page * kv_heads + kvh) * page_size + (j % page_size)) * (size_t)d + e0;
-      float kv[8];
-      if (live) ld8(k_cache + base, kv);
-      else
+    // four of the wave's keys at a time, their loads first: a loop that waits for memory once a key costs a
+    // round trip per key (a key past the end reads the last one again and stores nothing)
+    const int stride = ATT_WAVES * TPW;
+    for (int t0 = wave * TPW + slot; t0 < count; t0 += 4 * stride) {
+      float kv[4][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) kv[e] = 0.f;
+      for (int u = 0; u < 4; ++u) {
+        const int j = begin + min(t0 + u * stride, count - 1);
+        const size_t page = table[j / page_size];
+        const size_t base = ((page * kv_heads + kvh) * page_size + (j % page_size)) * (size_t)d + e0;
+        if (live) ld8(k_cache + base, kv[u]);
+        else
 #pragma unroll
-      for (int h = 0; h < GT; ++h) {
-        float dot = 0.f;
+          for (int e = 0; e < 8; ++e) kv[u][e] = 0.f;
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) dot += qv[h][e] * kv[e];
-        for (int o = TG >> 1; o > 0; o >>= 1) dot += __shfl_xor(dot, o, QIL_WAVE);
-        if (sub == 0) scores[h * P + t] = dot * scale;
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * stride;
+#pragma unroll
+        for (int h = 0; h < GT; ++h) {
+          float dot = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dot += qv[h][e] * kv[u][e];
+          for (int o = TG >> 1; o > 0; o >>= 1) dot += __shfl_xor(dot, o, QIL_WAVE);
+          if (sub == 0 && t < count) scores[h * P + t] = dot * scale;
+        }
       }
     }
     __syncthreads();
@@ -110,19 +120,28 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
     for (int h = 0; h < GT; ++h)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-    for (int t = wave * TPW + slot; t < count; t += ATT_WAVES * TPW) {
-      const int j = begin + t;
-      const size_t page = table[j / page_size];
-      // V is [pages, kv_heads, d, page_size]: this key's elements lie page_size apart
-      const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + e0) * page_size + (j % page_size);
-      float vv[8];
+    for (int t0 = wave * TPW + slot; t0 < count; t0 += 4 * stride) {      // four keys at a time, as above
+      float vv[4][8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vv[e] = live ? ld(column + (size_t)e * page_size) : 0.f;
+      for (int u = 0; u < 4; ++u) {
+        const int j = begin + min(t0 + u * stride, count - 1);
+        const size_t page = table[j / page_size];
+        // V is [pages, kv_heads, d, page_size]: this key's elements lie page_size apart
+        const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + e0) * page_size + (j % page_size);
 #pragma unroll
-      for (int h = 0; h < GT; ++h) {
-        const float p = scores[h * P + t];
+        for (int e = 0; e < 8; ++e) vv[u][e] = live ? ld(column + (size_t)e * page_size) : 0.f;
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] += p * vv[e];
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * stride;
+        if (t < count) {
+#pragma unroll
+          for (int h = 0; h < GT; ++h) {
+            const float p = scores[h * P + t];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] += p * vv[u][e];
+          }
+        }
       }
     }
     // sum over the token slots of the wave, then over the waves (fixed order)
