@@ -91,7 +91,14 @@ def _code(dtype):
         raise UnsupportedShape(f'kernels exist for float32 and bfloat16, not {dtype}') from None
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def _stream():
+    """The current stream's handle.  (torch's direct accessor where it has one: building a Stream object for
+    every launch cost a quarter of a small model's step on the host.)"""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
