@@ -47,30 +47,31 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   bf16_t* tiles = reinterpret_cast<bf16_t*>(lds_raw);
   int* pages = reinterpret_cast<int*>(tiles + (TWO ? 2 : 1) * TILE_ELEMS);   // the block-table entries this block needs
 
-  const int seq = blockIdx.y;
-  const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
-  if (n < 2) return;
-  const int RT = 4 / GH;
-  const int block_rows = 16 * RB * RT;
-  // Which row tile and which (kv head, head chunk) this block takes.  Blocks go to the 8 XCDs in turn, each with
-  // an L2 of its own: with one sequence and a number of (kv head, chunk) pairs that 256 is a multiple of, block
-  // id takes pair id % pairs, so that an XCD sees the keys and values of few kv heads (one, with 8 of them) and
-  // its L2 holds them; and of the row tiles, consecutive groups of 256 blocks walk them in opposite directions,
-  // so that the two blocks a CU holds make one long and one short pass over the keys.
-  int across, pair = blockIdx.z;
-  const int pairs = gridDim.z, tiles_x = gridDim.x;
-  if (gridDim.y == 1 && 256 % pairs == 0) {
-    const int id = blockIdx.x + tiles_x * blockIdx.z;
-    pair = id % pairs;
-    // places in spans of 2 * (256 / pairs): the first half of a span takes its upper tiles from the top down, the
-    // second half its lower tiles from the bottom up (the last span may be shorter)
-    const int place = id / pairs, span = 2 * (256 / pairs), base = place / span * span;
+  // Which sequence, row tile and (kv head, head chunk) this block takes.  Blocks go to the 8 XCDs in turn, each
+  // with an L2 of its own: when 256 is a multiple of the number of (sequence, kv head, chunk) triples, block id
+  // takes triple id % triples, so that an XCD sees the keys and values of few kv heads (one, with one sequence
+  // and 8 of them) and its L2 holds them; and of the row tiles, consecutive groups of 256 blocks walk them in
+  // opposite directions, so that the two blocks a CU holds make one long and one short pass over the keys.
+  int across, seq = blockIdx.y, pair = blockIdx.z;
+  const int triples = gridDim.y * gridDim.z, tiles_x = gridDim.x;
+  if (256 % triples == 0) {
+    const int id = blockIdx.x + tiles_x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int triple = id % triples;
+    seq = triple % gridDim.y;
+    pair = triple / gridDim.y;
+    // places in spans of 2 * (256 / triples): the first half of a span takes its upper tiles from the top down,
+    // the second half its lower tiles from the bottom up (the last span may be shorter)
+    const int place = id / triples, span = 2 * (256 / triples), base = place / span * span;
     const int size = min(span, tiles_x - base), idx = place - base, upper = (size + 1) / 2;
     across = base + (idx < upper ? size - 1 - idx : idx - upper);
   } else {
     const int linear = tiles_x * (blockIdx.y + gridDim.y * blockIdx.z);
     across = ((linear >> 8) & 1) ? (int)blockIdx.x : tiles_x - 1 - (int)blockIdx.x;
   }
+  const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
+  if (n < 2) return;
+  const int RT = 4 / GH;
+  const int block_rows = 16 * RB * RT;
   const int tile_row0 = across * block_rows;
   if (tile_row0 >= n) return;
   const int kvh = pair / chunks, chunk = pair % chunks;
