@@ -32,15 +32,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define FAST_PAD 8                                         // LDS row padding in elements
 #define FAST_TABLE_MAX 4096                                // block-table entries of a sequence kept in LDS
 
-template <int D, int RB>
-__global__ void __launch_bounds__(FAST_THREADS, 2)
+template <int D, int RB, int WAVES>
+__global__ void __launch_bounds__(WAVES * QIL_WAVE, WAVES == 4 ? 2 : 1)
 attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                       const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
                       int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift) {
+  constexpr int FAST_THREADS_ = WAVES * QIL_WAVE;
   constexpr int BK = FAST_BK, QFRAGS = D / 32, DTILES = D / 16, SUB = BK / 16;
   constexpr int K_ROW = D + FAST_PAD, V_ROW = BK + FAST_PAD;
-  constexpr int K_ITERS = BK * (D / 8) / FAST_THREADS, V_ITERS = D * (BK / 8) / FAST_THREADS;
+  constexpr int K_ITERS = BK * (D / 8) / FAST_THREADS_, V_ITERS = D * (BK / 8) / FAST_THREADS_;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   constexpr bool TWO = D <= 128;                           // two tiles in LDS
   constexpr int TILE_ELEMS = BK * K_ROW + D * V_ROW;       // K [BK][K_ROW] (rows in score-tile order), then V^T [D][V_ROW]
@@ -70,7 +71,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   }
   const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
   if (n < 2) return;
-  const int RT = 4 / GH;
+  const int RT = WAVES / GH;
   const int block_rows = 16 * RB * RT;
   const int tile_row0 = across * block_rows;
   if (tile_row0 >= n) return;
@@ -94,7 +95,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   const int first_page = first_tile >> ps_shift, last_page = (key_end - 1) >> ps_shift;
   {
     const int* table = block_tables + (size_t)seq * table_stride;
-    for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS) pages[i] = table[first_page + i];
+    for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS_) pages[i] = table[first_page + i];
   }
 
   int my_row[RB], my_pos[RB];
@@ -170,7 +171,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     uint32_t k_at[K_ITERS], v_at[V_ITERS];
 #pragma unroll
     for (int it = 0; it < K_ITERS; ++it) {                   // all the table entries first, then all the loads
-      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int idx = threadIdx.x + it * FAST_THREADS_;
       const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
       const int key = min(max(k0 + kl, key_begin), key_end - 1);     // clamped onto a needed key; zeroed when published
       k_page[it] = pages[(key >> ps_shift) - first_page];
@@ -178,7 +179,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     }
 #pragma unroll
     for (int it = 0; it < V_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int idx = threadIdx.x + it * FAST_THREADS_;
       const int grp = idx / D, dim = idx % D;
       const int key = min(max(k0 + grp * 8, key_begin & ~7), (key_end - 1) & ~7);
       v_page[it] = pages[(key >> ps_shift) - first_page];
@@ -200,7 +201,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     const bool inside = k0 >= key_begin && k0 + BK <= key_end;        // no key of the tile needs zeroing
 #pragma unroll
     for (int it = 0; it < K_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int idx = threadIdx.x + it * FAST_THREADS_;
       const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
       const int key = k0 + kl;
       const bool valid = inside || (key >= key_begin && key < key_end);
@@ -210,7 +211,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     }
 #pragma unroll
     for (int it = 0; it < V_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS;
+      const int idx = threadIdx.x + it * FAST_THREADS_;
       const int grp = idx / D, dim = idx % D;
       uint4 raw = v_reg[it];
       if (!inside) {       // zero what lies outside [key_begin, key_end): never written, or someone else's
@@ -438,15 +439,15 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   }
 }
 
-template <int D, int RB>
+template <int D, int RB, int WAVES>
 static int launch_fast(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                        int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s) {
   const int g = heads / kv_heads;
-  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
+  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = WAVES / GH;
   const size_t lds = (D <= 128 ? 2 : 1) * ((size_t)FAST_BK * (D + FAST_PAD) + (size_t)D * (FAST_BK + FAST_PAD)) * sizeof(bf16_t) +
                      (size_t)table_stride * sizeof(int);
-  auto kernel = attn_tile_bf16_kernel<D, RB>;
+  auto kernel = attn_tile_bf16_kernel<D, RB, WAVES>;
   static size_t granted = 0;                     // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -457,11 +458,14 @@ static int launch_fast(const void* q, int q_stride, const void* k_cache, const v
   int ps_shift = -1;                                      // log2 of a power-of-two page size
   for (int b = 0; b < 30; ++b)
     if (page_size == (1 << b)) ps_shift = b;
-  hipLaunchKernelGGL(kernel, grid, dim3(FAST_THREADS), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+  hipLaunchKernelGGL(kernel, grid, dim3(WAVES * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                      (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
                      kv_heads, page_size, window, scale, GH, chunks, ps_shift);
   return (int)hipGetLastError();
 }
+
+static int tile_waves_override = 0;                       // tuning runs and tests: 4 or 8 forces the block size
+extern "C" void qil_attn_tile_waves(int waves) { tile_waves_override = waves; }
 
 // 1 if the kernel of this file takes the sizes (bfloat16 only).
 extern "C" int qil_attn_tile_bf16_takes(int d, int page_size, int table_stride) {
@@ -479,11 +483,21 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
       kv_heads * 2 > 65535)
     return -1;
   if (d == 64)
-    return launch_fast<64, 2>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
-                              n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+    return launch_fast<64, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                 n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+  // Head size 128: blocks of 8 waves (64 rows of 4 heads, or 128 of 2, ... share a staged tile of keys; one block
+  // a CU) once blocks of 4 waves would be four or more a CU: measured equal at 4 x 1024 tokens of 32 heads,
+  // 5 % faster at 4,096 tokens, 18 % at 8,192, and slower below (2,048 tokens: 81 against 80 us).
+  const int g128 = heads / kv_heads, gh128 = g128 >= 3 ? 4 : g128;
+  const long blocks4 = (long)((max_query + 32 * (4 / gh128) - 1) / (32 * (4 / gh128))) * n_seqs * kv_heads *
+                       ((g128 + gh128 - 1) / gh128);
+  const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 1024;
+  if (d == 128 && wide)
+    return launch_fast<128, 2, 8>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
   if (d == 128)
-    return launch_fast<128, 2>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
-                               n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
-  return launch_fast<256, 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
-                             n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+    return launch_fast<128, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+  return launch_fast<256, 1, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
 }

@@ -159,6 +159,8 @@ def _declare(lib):
     lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_gemm_bf16_splits.argtypes = [i, i, i]
     lib.qil_gemm_bf16_splits.restype = i
+    lib.qil_attn_tile_waves.argtypes = [i]
+    lib.qil_attn_tile_waves.restype = None
     lib.qil_gemm_bf16_streams.argtypes = [i, i, i, i]
     lib.qil_gemm_bf16_streams.restype = i
     lib.qil_gemm_bf16_unmerged.argtypes = [p, p, p, p, i, i, i, i, i, i, i, i, p]

@@ -483,6 +483,22 @@ def test_prompt_portions_against_float64(ops, dtype, lengths, chunks, page_size,
     mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, None, scale=d ** -0.5)
 
 
+@pytest.mark.parametrize('lengths,chunks,heads,kv_heads,window', [
+    ([700, 90, 33], [700, 31, 33], 16, 4, None),                # g = 4: 64 rows of 4 heads a block
+    ([513, 200], [300, 200], 8, 4, None),                       # g = 2: 128 rows of 2 heads
+    ([400], [400], 4, 4, None),                                 # g = 1: 256 rows of one head
+    ([600, 64], [600, 17], 10, 2, 100),                         # g = 5: two chunks of heads, a window
+])
+def test_prompt_attention_in_blocks_of_eight_waves(ops, lengths, chunks, heads, kv_heads, window):
+    """Long prompts of head size 128 run in blocks of 8 waves; forced here on short ones, against float64."""
+    lib = ops.library.load()
+    lib.qil_attn_tile_waves(8)
+    try:
+        mixed_attention_case(ops, torch.bfloat16, lengths, chunks, 16, 128, heads, kv_heads, window, scale=128 ** -0.5)
+    finally:
+        lib.qil_attn_tile_waves(0)
+
+
 def test_one_far_key_among_hundreds(ops):
     """Scale one early key so its score dominates: the output must be that key's value, from the
     right page and the right kv head (h // g, not h % kv_heads)."""
