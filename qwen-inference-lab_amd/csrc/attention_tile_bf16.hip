@@ -37,7 +37,9 @@ __global__ void __launch_bounds__(WAVES * QIL_WAVE, WAVES == 4 ? 2 : 1)
 attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                       const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
-                      int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift) {
+                      int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift,
+                      float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P,
+                      int parts) {
   constexpr int FAST_THREADS_ = WAVES * QIL_WAVE;
   constexpr int BK = FAST_BK, QFRAGS = D / 32, DTILES = D / 16, SUB = BK / 16;
   constexpr int K_ROW = D + FAST_PAD, V_ROW = BK + FAST_PAD;
@@ -69,6 +71,10 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     const int linear = tiles_x * (blockIdx.y + gridDim.y * blockIdx.z);
     across = ((linear >> 8) & 1) ? (int)blockIdx.x : tiles_x - 1 - (int)blockIdx.x;
   }
+  // parts > 1 (a few row tiles against a long context): grid.z also counts the parts of P keys, and a block
+  // leaves float32 partial results (the layout of the split-context row kernels) for the merge kernel
+  const int part = pair / (kv_heads * chunks);
+  pair -= part * (kv_heads * chunks);
   const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
   if (n < 2) return;
   const int RT = WAVES / GH;
@@ -87,8 +93,13 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
 
   const int rows_in_block = min(block_rows, n - tile_row0);
   const int pos_first = start + tile_row0;
-  const int key_end = pos_first + rows_in_block;                       // last position + 1
-  const int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  int key_end = pos_first + rows_in_block;                             // last position + 1
+  int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  if (parts > 1) {                                                     // P is a multiple of the tile's keys
+    key_begin = max(key_begin, part * P);
+    key_end = min(key_end, (part + 1) * P);
+    if (key_begin >= key_end) return;                                  // no row of the block sees a key of this part
+  }
   const int first_tile = key_begin / BK * BK;
 
   // block-table entries of [first_tile, key_end) into LDS
@@ -414,6 +425,22 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   if constexpr (WIDE) {
     const float total = wide_l + __shfl_xor(wide_l, 32, QIL_WAVE);
     if (!wide_valid) return;
+    if (parts > 1) {
+      // acc [row, head, part, d] unnormalised, m (the maximum in the exponent's units) and l [row, head, part]; a row
+      // that sees no key of this part leaves m = -inf, l = 0 in a cell the merge does not read
+      const size_t cell = ((size_t)(q0 + wide_row) * heads + head) * parts + part;
+#pragma unroll
+      for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<float4*>(part_acc + cell * D + 32 * t + 8 * j + 4 * half) =
+              make_float4(ow[t][4 * j], ow[t][4 * j + 1], ow[t][4 * j + 2], ow[t][4 * j + 3]);
+      if (half == 0) {
+        part_m[cell] = wide_m == -INFINITY ? -INFINITY : wide_m * scale;
+        part_l[cell] = total;
+      }
+      return;
+    }
     const float inv = 1.f / total;
     bf16_t* orow = out + ((size_t)(q0 + wide_row) * heads + head) * D;
 #pragma unroll
@@ -442,7 +469,8 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
 template <int D, int RB, int WAVES>
 static int launch_fast(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
-                       int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s) {
+                       int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s,
+                       float* workspace = nullptr, int total_rows = 0, int P = 0, int parts = 1) {
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = WAVES / GH;
   const size_t lds = (D <= 128 ? 2 : 1) * ((size_t)FAST_BK * (D + FAST_PAD) + (size_t)D * (FAST_BK + FAST_PAD)) * sizeof(bf16_t) +
@@ -454,13 +482,15 @@ static int launch_fast(const void* q, int q_stride, const void* k_cache, const v
     if (e != hipSuccess) return (int)e;
     granted = lds;
   }
-  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks);
+  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks * parts);
+  float* part_m = workspace ? workspace + (size_t)total_rows * heads * parts * D : nullptr;
+  float* part_l = part_m ? part_m + (size_t)total_rows * heads * parts : nullptr;
   int ps_shift = -1;                                      // log2 of a power-of-two page size
   for (int b = 0; b < 30; ++b)
     if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                      (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
-                     kv_heads, page_size, window, scale, GH, chunks, ps_shift);
+                     kv_heads, page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts);
   return (int)hipGetLastError();
 }
 
@@ -500,4 +530,48 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
                                   n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
   return launch_fast<256, 1, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                 n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+}
+
+// Keys in parts: a portion of a prompt deep in a long context is a few row tiles, each with thousands of keys ahead of
+// it, and fewer blocks than the chip has CUs.  Returns the number of parts to cut the keys into (1: do not) and
+// their size in *P: about two blocks a CU, parts of at least 256 keys, at most 16 of them.
+extern "C" int qil_attn_tile_parts(int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
+                                   int table_stride, int max_context, int* P) {
+  *P = 0;
+  if ((d != 64 && d != 128) || !qil_attn_tile_bf16_takes(d, page_size, table_stride) || heads % kv_heads ||
+      max_query < 2 || max_context < 1024)
+    return 1;
+  const int g = heads / kv_heads, gh = g >= 3 ? 4 : g, rows = 32 * (4 / gh);
+  const long blocks = (long)((max_query + rows - 1) / rows) * n_seqs * kv_heads * ((g + gh - 1) / gh);
+  if (blocks >= 256) return 1;
+  const int want = (int)min(16L, (512 + blocks - 1) / blocks);
+  int part = ((max_context + want - 1) / want + FAST_BK - 1) / FAST_BK * FAST_BK;
+  part = max(part, 256);
+  const int parts = (max_context + part - 1) / part;
+  if (parts < 2) return 1;
+  *P = part;
+  return parts;
+}
+
+// qil_attn_tile_bf16 with the keys in `parts` parts of P keys (P a multiple of 64, head size 64 or 128): every row
+// of a sequence of two or more rows gets float32 partial results in `workspace` (qil_attn_rows_workspace bytes for
+// all `total_rows` rows of the step, indexed by the step's row), which qil_attn_merge then turns into `out`.  The
+// cells of rows that are alone in their sequence stay unwritten.
+extern "C" int qil_attn_tile_bf16_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                        const int* block_tables, int table_stride, const int* cu_seqlens,
+                                        const int* seq_starts, void* workspace, int total_rows, int n_seqs,
+                                        int max_query, int heads, int kv_heads, int d, int page_size, int window,
+                                        float scale, int P, int parts, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if ((d != 64 && d != 128) || !qil_attn_tile_bf16_takes(d, page_size, table_stride) || heads % kv_heads ||
+      n_seqs > 65535 || parts < 2 || P < FAST_BK || P % FAST_BK || !workspace || total_rows < 1 ||
+      (long)kv_heads * 2 * parts > 65535)
+    return -1;
+  if (d == 64)
+    return launch_fast<64, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
+                                 nullptr, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
+                                 (float*)workspace, total_rows, P, parts);
+  return launch_fast<128, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
+                                nullptr, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
+                                (float*)workspace, total_rows, P, parts);
 }

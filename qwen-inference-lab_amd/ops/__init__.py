@@ -11,6 +11,8 @@ kernel library cannot be built or loaded every op raises.
 Tensors: ``T`` is the model's dtype (float32 or bfloat16).  The residual stream
 is float32.  Index tensors are int32.
 """
+import ctypes
+
 import torch
 
 from . import library
@@ -368,6 +370,23 @@ def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps,
     return out
 
 
+TILE_KEY_PARTS = None   # tests: (keys per part, parts) forces the tile kernel's key split where it takes the sizes
+
+
+def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context):
+    """(keys per part, parts) for the matrix-core tile kernel; parts == 1: the keys in one piece."""
+    if dtype != torch.bfloat16:
+        return 0, 1
+    part = ctypes.c_int(0)
+    parts = lib.qil_attn_tile_parts(n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context,
+                                    ctypes.byref(part))
+    if TILE_KEY_PARTS is not None and head_dim in (64, 128) and lib.qil_attn_tile_bf16_takes(head_dim, page_size,
+                                                                                              table_stride):
+        part = ctypes.c_int(TILE_KEY_PARTS[0])
+        parts = max(TILE_KEY_PARTS[1], -(-max_context // part.value))
+    return part.value, parts
+
+
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
                     unmerged=False):
@@ -398,10 +417,25 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
         if block_tables.shape[0] != n_seqs:
             raise ValueError('one block table row per sequence')
-        _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
-                                 block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
-                                 max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
-                                 _code(qkv.dtype), _stream()), 'attn_tile')
+        part, parts = tile_key_parts(lib, qkv.dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size,
+                                     block_tables.shape[1], max_context)
+        if parts > 1:
+            # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
+            # rows of the step: what the merge leaves in rows that are alone is overwritten below)
+            workspace = torch.empty(lib.qil_attn_rows_workspace(n, heads, head_dim, parts) // 4, dtype=torch.float32,
+                                    device=qkv.device)
+            _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                                                _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
+                                                _ptr(seq_starts), _ptr(workspace), n, n_seqs, max_query, heads,
+                                                kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
+                                                parts, _stream()), 'attn_tile_parts')
+            _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), n, heads, head_dim,
+                                      int(window or 0), part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
+        else:
+            _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+                                     block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
+                                     max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
+                                     _code(qkv.dtype), _stream()), 'attn_tile')
         if single_rows is None:
             raise ValueError('single_rows must list the rows that are alone when some sequence has several')
         _require(single_rows, 'single_rows', torch.int32)

@@ -499,6 +499,36 @@ def test_prompt_attention_in_blocks_of_eight_waves(ops, lengths, chunks, heads, 
         lib.qil_attn_tile_waves(0)
 
 
+@pytest.mark.parametrize('lengths,chunks,d,heads,kv_heads,window,split', [
+    ([700, 90, 33], [100, 1, 33], 128, 16, 4, None, (64, 2)),    # parts of one tile; a whole short prompt beside it
+    ([513, 200, 64], [70, 200, 1], 128, 8, 4, None, (128, 2)),   # a part's edge inside a portion's rows (512 | 513)
+    ([640], [129], 64, 4, 2, None, (192, 2)),                    # head size 64; a portion that starts on an edge
+    ([600, 64], [77, 17], 128, 10, 2, 100, (64, 3)),             # a window: the first parts hold nothing for a row
+    ([900], [2], 128, 8, 8, 300, (256, 2)),                      # two rows, g = 1
+    ([1030, 300], [130, 2], 64, 6, 2, 64, (64, 4)),              # g = 3, a window of one part's size
+])
+def test_prompt_portion_with_keys_in_parts(ops, monkeypatch, lengths, chunks, d, heads, kv_heads, window, split):
+    """A portion deep in a long context has its keys cut into parts that are merged afterwards; forced on short
+    contexts here, with edges of parts at and inside the portion's rows, against float64."""
+    monkeypatch.setattr(ops, 'TILE_KEY_PARTS', split)
+    mixed_attention_case(ops, torch.bfloat16, lengths, chunks, 16, d, heads, kv_heads, window, scale=d ** -0.5)
+
+
+@pytest.mark.parametrize('lengths,chunks,heads,kv_heads,window', [
+    ([2048], [128], 32, 8, None),
+    ([4000, 3000, 1500], [64, 1, 2], 16, 8, None),
+    ([5000], [130], 8, 2, 1100),
+])
+def test_prompt_portion_deep_in_a_long_context(ops, lengths, chunks, heads, kv_heads, window):
+    """The sizes at which the split is chosen by itself."""
+    lib = ops.library.load()
+    table_stride = -(-max(lengths) // 16)
+    part, parts = ops.tile_key_parts(lib, torch.bfloat16, len(lengths), max(chunks), heads, kv_heads, 128, 16,
+                                     table_stride, max(lengths))
+    assert parts > 1 and part % 64 == 0 and part * parts >= max(lengths)
+    mixed_attention_case(ops, torch.bfloat16, lengths, chunks, 16, 128, heads, kv_heads, window, scale=128 ** -0.5)
+
+
 def test_one_far_key_among_hundreds(ops):
     """Scale one early key so its score dominates: the output must be that key's value, from the
     right page and the right kv head (h // g, not h % kv_heads)."""
