@@ -713,12 +713,21 @@ static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
     if (sp > most) sp = most;
     while (sp > 1 && steps / sp < 8) --sp;
     if (sp < 1) sp = 1;
-    // up to 16 rows: the most splits not above that which the whole-line kernel takes (whole stages of 128
-    // columns, at least LINES_DEPTH of them), if there is such a number
+    // up to 16 rows: of the splits the whole-line kernel takes (whole stages of 128 columns, at least LINES_DEPTH
+    // of them; up to 32), the one whose blocks fill their rounds of 256 CUs best, less 1.5 % a split for what the
+    // consumer of the partial sums reads.  One round of 160 blocks or more counts as full: measured, 160, 192,
+    // 256, 400 and 1,000 blocks stream equally well, 128, 280 and 320 (a last round a quarter full or less) 10 to
+    // 15 % slower, and 80 blocks 50 % slower than 380.
     if (M <= 16 && K % 128 == 0) {
       int fit = 0;
-      for (int c = sp; c >= 1 && !fit; --c)
-        if (K % (128 * c) == 0 && K / (128 * c) >= LINES_DEPTH) fit = c;
+      double fit_score = 0;
+      for (int c = 1; c <= 32; ++c) {
+        if (K % (128 * c) || K / (128 * c) < LINES_DEPTH || lines_lds(M, K, c) > LINES_LDS_LIMIT) continue;
+        const long blocks = (long)column_blocks * c;
+        const long slots = blocks >= 160 && blocks <= 256 ? blocks : (blocks + 255) / 256 * 256;
+        const double score = (double)blocks / (double)slots - 0.015 * c;
+        if (!fit || score > fit_score) { fit = c; fit_score = score; }
+      }
       if (fit) sp = fit;
     }
   }
