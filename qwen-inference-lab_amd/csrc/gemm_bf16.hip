@@ -2,7 +2,7 @@
 //   C[M, N] = A[M, K] W[N, K]^T (+ bias[N]),  float32 accumulation.
 // Four kernels, all bound by reading W once: `stream` (this comment; any shape, bias, unaligned operands),
 // `lines` (up to 16 rows, W in whole cache lines, optional merge of attention parts into A), `chunks`
-// (17 to 64 rows, A through LDS in stages) and `gated` (gate and up products with SiLU in the epilogue).
+// (17 to 128 rows, A through LDS in stages) and `gated` (gate and up products with SiLU in the epilogue).
 // Both operands have K contiguous (qil/model.py:32-40).  The product is bound by streaming W once
 // from HBM; A is small and would be re-read from L2 by every block, so the work is cut into wide,
 // short pieces: a block owns 128 * NT rows of W (8 waves, each 16 * NT rows) and ONE of `splits`
@@ -333,14 +333,15 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// The whole-line product for 17 to 64 rows of A and any length of K.  A does not stay in LDS as a whole
+// The whole-line product for 17 to 128 rows of A and any length of K.  A does not stay in LDS as a whole
 // slice: it passes through it one stage (128 columns) at a time, in two slots that the block's threads
 // fill in turn, from registers that are loaded three stages ahead, as W's are.  One barrier a stage: the
 // stage's slot has been written before it and the other slot may be written after it.  All waves of a
 // block are at the same stage, so the walk through K starts at a column of the block's (not the wave's) own.
 // MT: 16-row tiles of A (M <= 16 MT); every W fragment read from the buffer serves MT products.
-// Takes 16 < M <= 64, K a multiple of 128 per split with at least 3 stages, 16-byte aligned operands, no bias.
+// Takes 16 < M <= 128, K a multiple of 128 per split with at least 3 stages, 16-byte aligned operands, no bias.
 #define CHUNK_ROW (128 + GEMM_LDS_PAD)
+#define CHUNKS_MOST_ROWS 128
 
 template <typename OUT, int MT>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
@@ -457,7 +458,7 @@ gemm_bf16_chunks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
 }
 
 static bool chunks_takes(const void* A, const void* W, const float* bias, int M, int N, int K, int splits) {
-  return !bias && M > 16 && M <= 64 && N >= 1 && splits >= 1 && K % (128 * splits) == 0 &&
+  return !bias && M > 16 && M <= CHUNKS_MOST_ROWS && N >= 1 && splits >= 1 && K % (128 * splits) == 0 &&
          K / (128 * splits) >= LINES_DEPTH && (((uintptr_t)A | (uintptr_t)W) % 16) == 0;
 }
 
@@ -490,7 +491,9 @@ static int launch_chunks_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, 
 template <typename OUT>
 static int launch_chunks(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
   if (M <= 32) return launch_chunks_tiles<OUT, 2>(A, W, C, M, N, K, splits, s);
-  return launch_chunks_tiles<OUT, 4>(A, W, C, M, N, K, splits, s);
+  if (M <= 64) return launch_chunks_tiles<OUT, 4>(A, W, C, M, N, K, splits, s);
+  if (M <= 96) return launch_chunks_tiles<OUT, 6>(A, W, C, M, N, K, splits, s);
+  return launch_chunks_tiles<OUT, 8>(A, W, C, M, N, K, splits, s);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -737,16 +740,20 @@ static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
 
 // How many ways the product will be split over K when partial sums are allowed.
 extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
-  if (M > 16 && M <= 64 && K % 128 == 0 && K / 128 >= LINES_DEPTH) return chunks_splits(N, K);
+  if (M > 16 && M <= CHUNKS_MOST_ROWS && K % 128 == 0 && K / 128 >= LINES_DEPTH) return chunks_splits(N, K);
   int code, splits;
   plan(M, N, K, true, &code, &splits);
   return splits;
 }
 
-// 1 if a product with 17 to 64 rows has a weight-streaming kernel here (K a multiple of 128 of at least 384, no
-// bias; operands 16-byte aligned, which the call checks); products of up to 16 rows always have one.
+// 1 if a product with 17 to 128 rows should run on the weight-streaming kernel here (K a multiple of 128 of at
+// least 384, no bias; operands 16-byte aligned, which the call checks); products of up to 16 rows always do.
+// 65 to 128 rows: only products of at most 64 column tiles (N <= 8192), which the split over K spreads over
+// the CUs; measured at 128 rows and 8B layer sizes against the GPU BLAS: 21 us against 26 (q/k/v), 16 against
+// 24 (attention output), 33 against 67 (down), but 57 against 49 for the 192 tiles of gate/up.
 extern "C" int qil_gemm_bf16_streams(int M, int N, int K, int has_bias) {
   if (M <= 16) return 1;
+  if (M > 64 && N > 64 * 16 * LINES_WAVES) return 0;
   return chunks_takes(nullptr, nullptr, has_bias ? (const float*)1 : nullptr, M, N, K, 1);
 }
 

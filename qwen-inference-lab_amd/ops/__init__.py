@@ -21,8 +21,9 @@ from . import library
 STREAM_GEMM_MAX_ROWS = 16
 # ... and up to this many rows where K is a multiple of 128 (at least 384) and there is no bias: the kernel that
 # passes A through LDS in stages.  Measured at 64 rows and 8B layer sizes against the GPU BLAS: 41 us against 47
-# (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).
-STREAM_GEMM_MOST_ROWS = 64
+# (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
+# the library says which products it takes (those of few column tiles).
+STREAM_GEMM_MOST_ROWS = 128
 # Keys per split of the row attention kernel.
 ATTENTION_PART = 256
 # Blocks the matrix-core decode kernel aims for (256 CUs, 8 waves a block; measured best at 8 rows x 2048 keys).
