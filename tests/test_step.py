@@ -239,6 +239,71 @@ def test_graph_replays_equal_eager_launches(model_folder, dtype):
     torch.testing.assert_close(got, expected[5:13], **TOLERANCE[dtype])
 
 
+def random_configuration(r):
+    """Every size and option drawn at random: head sizes in steps of 16 up to 256, one to eight kv heads with
+    groups of one to sixteen, widths and vocabularies that are no powers of two, biases, tied or own head."""
+    kv, group = r.choice([1, 1, 2, 2, 3, 4, 5, 8]), r.choice([1, 2, 3, 4, 5, 6, 7, 8, 16])
+    return dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=r.randrange(50, 3000),
+                hidden_size=r.choice([2, 4, 8]) * r.randrange(9, 160),
+                intermediate_size=r.choice([2, 8, 16]) * r.randrange(5, 90), num_hidden_layers=r.randrange(1, 4),
+                num_attention_heads=kv * group, num_key_value_heads=kv,
+                head_dim=r.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256]), max_position_embeddings=2048,
+                rms_norm_eps=r.choice([1e-6, 1e-5, 3e-4]), rope_theta=r.choice([1e4, 5e5, 1e6]),
+                attention_bias=r.random() < 0.3, tie_word_embeddings=r.random() < 0.5, hidden_act='silu',
+                eos_token_id=None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('seed', range(12))
+def test_random_configurations_in_mixed_batches(model_folder, seed, dtype):
+    """Configurations drawn at random, six short prompts and one of hundreds of tokens in portions of 1 to 130
+    tokens, up to four live, pages reused, the pool full of NaN.  The logits of these models are not all of
+    size 1 (widths up to 1,272), so the error is measured against the largest logit of the request."""
+    r = random.Random(seed)
+    config, page_size = random_configuration(r), r.choice([3, 4, 8, 16, 16, 32])
+    folder, weights = model_folder(config, seed)
+    model = load_model(folder, dtype=dtype, device='cuda')
+    lengths = [r.randrange(1, 90) for _ in range(6)] + [r.randrange(200, 700)]
+    prompts = {i: tokens_for(config, n, 1000 * seed + i) for i, n in enumerate(lengths)}
+    pages = sum(-(-n // page_size) for n in sorted(lengths)[-4:]) + 1
+    runner = ModelRunner(model, num_pages=pages, page_size=page_size, max_requests=4)
+    poison(runner)
+    waiting, live, done = list(prompts), {}, {}
+    while waiting or live:
+        while waiting and len(live) < 4:
+            need = -(-len(prompts[waiting[0]]) // page_size)
+            if sum(-(-len(prompts[i]) // page_size) for i in live) + need > pages:
+                break
+            i = waiting.pop(0)
+            assert runner.admit(i)
+            live[i] = 0
+        order = list(live)
+        r.shuffle(order)
+        entries = []
+        for i in order:
+            left = len(prompts[i]) - live[i]
+            size = 1 if left <= 3 or r.random() < 0.3 else min(left, r.choice([2, 3, 5, 8, 17, 40, 130]))
+            entries.append(StepEntry(i, tuple(prompts[i][live[i]:live[i] + size]), tuple(range(size))))
+        logits = runner.step(entries).cpu()
+        at = 0
+        for entry in entries:
+            size = len(entry.tokens)
+            done.setdefault(entry.request, []).append(logits[at:at + size])
+            at += size
+            live[entry.request] += size
+            if live[entry.request] == len(prompts[entry.request]):
+                runner.release(entry.request)
+                del live[entry.request]
+        runner.cache.check()
+    assert runner.cache.free_pages == [pages]
+    for i in prompts:
+        got, want = torch.cat(done[i]), plain.logits(prompts[i], weights, config)
+        assert torch.isfinite(got).all()
+        largest = max(1.0, want.abs().max().item())
+        assert (got - want).abs().max().item() <= TOLERANCE[dtype]['atol'] * largest, (config, page_size, i)
+
+
 @pytest.mark.parametrize('backend', BACKENDS, indirect=True)
 def test_schedule_with_a_repeated_layer_and_a_shared_cache(model_folder, backend):
     """The run order is data: layer 0 runs twice (each run with a cache of its own) and the last entry
