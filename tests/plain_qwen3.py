@@ -9,8 +9,6 @@ repository root) whose formula it restates.
 dict of config.json.  `dtype` is the arithmetic type: float32 (default),
 float64 for tight pins, or bfloat16 to follow the reference's rounding places.
 """
-import math
-
 import torch
 
 

@@ -3,7 +3,7 @@ import pytest
 import torch
 
 from qil_amd.cache import CacheManager
-from qil_amd.engine import Engine, Request, Scheduler, StepEntry
+from qil_amd.engine import Engine, Request, Scheduler
 from qil_amd.parts import KVNeed
 
 
