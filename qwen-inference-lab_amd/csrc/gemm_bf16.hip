@@ -549,15 +549,37 @@ gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
 #pragma unroll
     for (int u = 0; u < 4; ++u) w[u] = *reinterpret_cast<const u32x4*>(gate_source[u] + offset + at);
   };
-  // A first (its wait would otherwise cover W's first stages), then W's first two stages
-  for (int idx = threadIdx.x; idx < a_rows * (K / 8); idx += blockDim.x) {
-    const int m = idx / (K / 8), c = (idx - m * (K / 8)) * 8;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (m < M) v = *reinterpret_cast<const uint4*>(A + (size_t)m * K + c);
-    *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+  // A long A (more than two 16-byte pieces a thread): W's first two stages are requested first, then A is staged
+  // four pieces a thread at a time with all four loads before the first store; a loop of load, wait, store pays
+  // a round trip to L2 for every piece, six of them at K = 4096.  Measured in one process, 8 rows: 36.9 -> 35.6 us
+  // at 8B sizes, 26.8 -> 22.2 at 4B sizes.  Rows past M repeat row M - 1 and pieces past the end repeat the last
+  // one (a load under a condition would make every later wait a wait for all loads): their products are rows
+  // of D that are never stored.  A short A keeps the old order, which is 0.5 us faster at 0.6B sizes.
+  const int per_row = K / 8, total = a_rows * per_row;
+  if (total <= 2 * (int)blockDim.x) {                       // a short A: one or two pieces a thread, A first
+    for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+      const int m = idx / per_row, c = (idx - m * per_row) * 8;
+      *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = *reinterpret_cast<const uint4*>(A + (size_t)min(m, M - 1) * K + c);
+    }
+    request(g0, 0, 0); request(u0, up_offset, 0);
+    request(g1, 0, 1); request(u1, up_offset, 1);
+  } else {
+    request(g0, 0, 0); request(u0, up_offset, 0);           // the host sees to stages >= 2
+    request(g1, 0, 1); request(u1, up_offset, 1);
+    for (int base = threadIdx.x; base < total; base += 4 * blockDim.x) {
+      uint4 v[4];
+      int to[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = min(base + j * (int)blockDim.x, total - 1);
+        const int m = idx / per_row, c = (idx - m * per_row) * 8;
+        v[j] = *reinterpret_cast<const uint4*>(A + (size_t)min(m, M - 1) * K + c);
+        to[j] = m * row_width + c;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(a_lds + to[j]) = v[j];
+    }
   }
-  request(g0, 0, 0); request(u0, up_offset, 0);             // the host sees to stages >= 2
-  request(g1, 0, 1); request(u1, up_offset, 1);
   __syncthreads();
 
   f32x4 gate = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
