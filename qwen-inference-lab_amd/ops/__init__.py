@@ -418,8 +418,12 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
         if block_tables.shape[0] != n_seqs:
             raise ValueError('one block table row per sequence')
-        part, parts = tile_key_parts(lib, qkv.dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size,
-                                     block_tables.shape[1], max_context)
+        if single_rows is None:
+            raise ValueError('single_rows must list the rows that are alone when some sequence has several')
+        _require(single_rows, 'single_rows', torch.int32)
+        # sequences of one row leave their blocks at once: only the others count for how full the chip is
+        part, parts = tile_key_parts(lib, qkv.dtype, max(1, n_seqs - single_rows.shape[0]), max_query, heads, kv_heads,
+                                     head_dim, page_size, block_tables.shape[1], max_context)
         if parts > 1:
             # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
             # rows of the step: what the merge leaves in rows that are alone is overwritten below)
@@ -437,9 +441,6 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                                      block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
                                      max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
                                      _code(qkv.dtype), _stream()), 'attn_tile')
-        if single_rows is None:
-            raise ValueError('single_rows must list the rows that are alone when some sequence has several')
-        _require(single_rows, 'single_rows', torch.int32)
         rows = single_rows.shape[0]
     else:
         single_rows, rows = None, n

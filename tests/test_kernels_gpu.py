@@ -518,13 +518,14 @@ def test_prompt_portion_with_keys_in_parts(ops, monkeypatch, lengths, chunks, d,
     ([2048], [128], 32, 8, None),
     ([4000, 3000, 1500], [64, 1, 2], 16, 8, None),
     ([5000], [130], 8, 2, 1100),
+    ([3000] + [900] * 12, [128] + [1] * 12, 32, 8, None),       # one portion beside a dozen decoded rows
 ])
 def test_prompt_portion_deep_in_a_long_context(ops, lengths, chunks, heads, kv_heads, window):
-    """The sizes at which the split is chosen by itself."""
+    """The sizes at which the split is chosen by itself (sequences of one row do not count as work)."""
     lib = ops.library.load()
     table_stride = -(-max(lengths) // 16)
-    part, parts = ops.tile_key_parts(lib, torch.bfloat16, len(lengths), max(chunks), heads, kv_heads, 128, 16,
-                                     table_stride, max(lengths))
+    part, parts = ops.tile_key_parts(lib, torch.bfloat16, sum(c > 1 for c in chunks), max(chunks), heads, kv_heads, 128,
+                                     16, table_stride, max(lengths))
     assert parts > 1 and part % 64 == 0 and part * parts >= max(lengths)
     mixed_attention_case(ops, torch.bfloat16, lengths, chunks, 16, 128, heads, kv_heads, window, scale=128 ** -0.5)
 
