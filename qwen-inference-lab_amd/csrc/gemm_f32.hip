@@ -106,7 +106,7 @@ sgemv_rows_kernel(const float* __restrict__ A, const float* __restrict__ W, cons
   }
 }
 
-// Few rows (decode), K % 4 == 0: the product is bound by streaming W once, so it is shaped like the
+// Few rows (decode, up to 64), K % 4 == 0: the product is bound by streaming W once, so it is shaped like the
 // bfloat16 streaming kernel (gemm_bf16.hip): a block owns 128 columns (8 waves x 16) and one of
 // `splits` ranges of K, stages its slice of A in LDS, and every wave streams its 16 rows of W from
 // global memory straight into v_mfma_f32_16x16x4_f32 operands: float32 inputs, float32 products and
@@ -117,6 +117,7 @@ sgemv_rows_kernel(const float* __restrict__ A, const float* __restrict__ W, cons
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 #define SF_WAVES 8
 #define SF_PAD 4
+#define SF_MOST_ROWS 64                                    // rows up to which the product streams W through the matrix cores
 
 template <int MT, int UNROLL>
 __global__ void __launch_bounds__(SF_WAVES * QIL_WAVE)
@@ -179,7 +180,7 @@ gemm_f32_stream_kernel(const float* __restrict__ A, const float* __restrict__ W,
 
 // Ways the few-row product will be split over K when partial sums are allowed (1: it is not split).
 extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
-  if (M > 16 || K % 4) return 1;
+  if (M > SF_MOST_ROWS || K % 4) return 1;
   const int column_blocks = (N + 127) / 128, steps = (K + 15) / 16;
   int sp = (768 + column_blocks - 1) / column_blocks;
   if (sp > 8) sp = 8;
@@ -187,24 +188,28 @@ extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
   return sp < 1 ? 1 : sp;
 }
 
-// C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs M <= 16,
+// C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs M <= 64,
 // K % 4 == 0 and no bias.
 extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
                             int splits, hipStream_t s) {
   if (M == 0 || N == 0) return 0;
   if (K < 1 || splits < 1) return -1;
-  const bool stream_ok = M <= 16 && K % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+  const bool stream_ok = M <= SF_MOST_ROWS && K % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
   if (splits > 1 && (!stream_ok || bias)) return -1;
   if (stream_ok) {
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;           // 16-row tiles of A a block keeps
     const int steps = (K + 15) / 16, steps_per_split = (steps + splits - 1) / splits;
     int chunk = steps_per_split * 16;
-    const int cap = (64 * 1024 / (16 * (int)sizeof(float)) - SF_PAD) / 64 * 64;      // columns per row within 64 KB
+    const int cap = (64 * 1024 / (16 * mt * (int)sizeof(float)) - SF_PAD) / 64 * 64;   // columns per row within 64 KB
     if (chunk > cap) chunk = cap;
     chunk = (chunk + 15) / 16 * 16;
-    const size_t lds = (size_t)16 * (chunk + SF_PAD) * sizeof(float);
+    const size_t lds = (size_t)16 * mt * (chunk + SF_PAD) * sizeof(float);
     dim3 grid((N + 127) / 128, 1, splits);
-    hipLaunchKernelGGL((gemm_f32_stream_kernel<1, 4>), grid, dim3(SF_WAVES * QIL_WAVE), lds, s, A, W, bias, C, M, N, K,
-                       steps_per_split, chunk);
+#define QIL_SF_LAUNCH(MT)                                                                                          \
+  hipLaunchKernelGGL((gemm_f32_stream_kernel<MT, 4>), grid, dim3(SF_WAVES * QIL_WAVE), lds, s, A, W, bias, C, M, N, K, \
+                     steps_per_split, chunk)
+    if (mt == 1) QIL_SF_LAUNCH(1); else if (mt == 2) QIL_SF_LAUNCH(2); else QIL_SF_LAUNCH(4);
+#undef QIL_SF_LAUNCH
     QIL_RETURN_LAUNCH_STATUS();
   }
   if (M <= 2 * SV_ROWS) {

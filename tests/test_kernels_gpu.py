@@ -107,6 +107,24 @@ def test_linear_float32(ops, m, n, k, bias):
     check(ops.linear(x, w, b), want, torch.float32, scale=4)
 
 
+@pytest.mark.parametrize('m,n,k', [(3, 1024, 4096), (16, 300, 2048), (20, 4096, 4096), (64, 1024, 3072), (33, 130, 516),
+                                   (48, 2000, 100), (65, 512, 1024)])
+def test_linear_float32_partial_sums(ops, m, n, k):
+    """Up to 64 rows the float32 product streams W through the float32 matrix-core instruction and may come
+    back split over K; with more rows it is one tensor."""
+    x, w = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5)
+    got = ops.linear(x, w, None, partials=True)
+    want = x.double() @ w.double().t()
+    if isinstance(got, ops.Partials):
+        assert m <= 64 and got.splits > 1 and got.shape == (m, n)
+        check(got.sum(), want, torch.float32, scale=4)
+    else:
+        assert m > 64 or ops.library.load().qil_gemm_f32_splits(m, n, k) == 1
+        check(got, want, torch.float32, scale=4)
+    if k >= 2048 and n <= 4096 and m <= 64:
+        assert isinstance(got, ops.Partials), 'a product with few columns and a long K should be split'
+
+
 @pytest.mark.parametrize('m,n,k', SHAPES)
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('bias', [False, True])
