@@ -183,25 +183,37 @@ __device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
   const int lo = u.window > 0 ? max(0, ctx - u.window) : 0;
   const int first = lo / u.P, last = (ctx - 1) / u.P;
   const size_t cell0 = ((size_t)m * u.heads + head) * u.parts;
-  // four parts at a time, all their loads first: a loop that waits for memory once per part would
-  // cost more than the merge kernel it replaces
+  // four parts at a time, all their loads first: a loop that waits for memory once per part would cost more
+  // than the merge kernel it replaces.  The first four parts' sums and values are asked for together with their
+  // maxima (they do not depend on the largest maximum, only their use does): one wait for up to four parts.
+  float mv[4], lv[4], part[4][8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int p = min(first + j, last);
+    mv[j] = u.m[cell0 + p];
+    lv[j] = u.l[cell0 + p];
+    ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
+  }
   float top = -INFINITY;
-  for (int p0 = first; p0 <= last; p0 += 4) {
-    float mv[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) mv[j] = u.m[cell0 + min(p0 + j, last)];
+  for (int j = 0; j < 4; ++j) top = fmaxf(top, mv[j]);
+  for (int p0 = first + 4; p0 <= last; p0 += 4) {
+    float more[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) top = fmaxf(top, mv[j]);
+    for (int j = 0; j < 4; ++j) more[j] = u.m[cell0 + min(p0 + j, last)];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) top = fmaxf(top, more[j]);
   }
   float denom = 0.f, numer[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int p0 = first; p0 <= last; p0 += 4) {
-    float mv[4], lv[4], part[4][8];
+    if (p0 != first) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int p = min(p0 + j, last);
-      mv[j] = u.m[cell0 + p];
-      lv[j] = u.l[cell0 + p];
-      ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
+      for (int j = 0; j < 4; ++j) {
+        const int p = min(p0 + j, last);
+        mv[j] = u.m[cell0 + p];
+        lv[j] = u.l[cell0 + p];
+        ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {                           // the order and the arithmetic of the merge kernel
