@@ -228,7 +228,8 @@ int qil_add_rmsnorm(float* stream, const void* delta, int delta_dtype, int split
   do {                                                                                                               \
     if (vec && width <= 256) QIL_NORM_VEC(TD, T, 64, 1);                                                             \
     else if (vec && width <= 1024) QIL_NORM_VEC(TD, T, 256, 1);                                                      \
-    else if (vec && width <= 4096) QIL_NORM_VEC(TD, T, 1024, 1);                                                     \
+    else if (vec && width <= 2048) QIL_NORM_VEC(TD, T, 512, 1);                                                      \
+    else if (vec && width <= 4096) QIL_NORM_VEC(TD, T, 512, 2);                                                      \
     else if (vec) QIL_NORM_VEC(TD, T, 1024, 2);                                                                      \
     else                                                                                                             \
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, T>), dim3(n_out), dim3(width >= 2048 ? 512 : width >= 512 ? 256 : 64), \
