@@ -178,9 +178,136 @@ gemm_f32_stream_kernel(const float* __restrict__ A, const float* __restrict__ W,
     }
 }
 
+// Up to 16 rows, K split into ranges of whole 64-column stages: W read in whole cache lines, as the bfloat16
+// whole-line kernel reads it (gemm_bf16.hip).  A load instruction takes 4 rows x 256 contiguous bytes (lane l:
+// row 4 u + l / 16, 16-byte piece l % 16), three stages of 16 rows x 64 columns are in flight in registers, and
+// a stage passes through a wave-private 4 KB LDS buffer that turns it into the operands of
+// v_mfma_f32_16x16x4_f32 (pieces stored at piece ^ row, so that writes and reads spread over all banks; LDS
+// operations of one wave complete in program order, so the buffer needs no barrier).  The block's slice of A
+// (8 or 16 rows) stays in LDS.  The fragment-layout kernel above touches half a cache line per row and load and
+// reaches about 3 TB/s at 8B layer sizes; this one streams at 4.3 to 5.6.  Always writes partial sums
+// C[split, M, N] (one split: the product itself).
+#define FL_WAVES 8
+#define FL_STAGE 64                                        // columns of a stage
+#define FL_PAD 4                                           // floats between rows of the slice of A
+#define FL_DEPTH 3                                         // stages of W in flight per wave
+#define FL_LDS_LIMIT (100 * 1024)
+
+__global__ void __launch_bounds__(FL_WAVES * QIL_WAVE)
+gemm_f32_lines_kernel(const float* __restrict__ A, const float* __restrict__ W, float* __restrict__ C, int M, int N,
+                      int K, int cols_per_split) {
+  extern __shared__ __align__(16) float fl_lds[];           // A slice [8 or 16][cols + pad], then the waves' buffers
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept (a power of two)
+  const int n0 = (blockIdx.x * FL_WAVES + wave) * 16, split = blockIdx.z;
+  const int k_begin = split * cols_per_split, stages = cols_per_split / FL_STAGE;
+  const int row_width = cols_per_split + FL_PAD;
+  float* a_lds = fl_lds;
+  float* buffer = fl_lds + a_rows * row_width + wave * (16 * FL_STAGE);
+
+  const int load_row = lane >> 4, piece = lane & 15;
+  const float* source[4];                                  // rows past N read a valid row and are never stored
+  int place[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    source[u] = W + (size_t)min(n0 + row, N - 1) * K + k_begin + piece * 4;
+    place[u] = row * FL_STAGE + ((piece ^ row) & 15) * 4;
+  }
+  // A slice first: its wait would otherwise cover the first stages of W as well
+  for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 4); idx += FL_WAVES * QIL_WAVE) {
+    const int m = idx / (cols_per_split / 4), c = (idx - m * (cols_per_split / 4)) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (m < M) v = *reinterpret_cast<const float4*>(A + (size_t)m * K + k_begin + c);
+    *reinterpret_cast<float4*>(a_lds + m * row_width + c) = v;
+  }
+  // every wave walks its K range from a start of its own and wraps around (waves that read the same columns
+  // of their rows at the same time load a few memory channels only)
+  const int turn = (n0 / 16) % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * FL_STAGE; };
+  f32x4v w0[4], w1[4], w2[4];                              // three stages, named so that none is indexed at run time
+  auto request = [&](f32x4v (&stage_w)[4], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const f32x4v*>(source[u] + at);
+  };
+  request(w0, 0);                                           // the host sees to stages >= 3
+  request(w1, 1);
+  request(w2, 2);
+  __syncthreads();
+
+  f32x4v acc = {0.f, 0.f, 0.f, 0.f};
+  // lanes past the kept rows read the rows again: their products are rows of D that are never stored
+  const float* a_row = a_lds + (r & (a_rows - 1)) * row_width + kb * 4;
+  auto pass = [&](const f32x4v (&stage_w)[4]) {            // registers -> buffer
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<f32x4v*>(buffer + place[u]) = stage_w[u];
+  };
+  auto multiply = [&](int stage) {
+    const int at = column(stage);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {                        // columns 16 s4 + 4 kb .. + 3 of the stage: four products
+      const f32x4v b = *reinterpret_cast<const f32x4v*>(buffer + r * FL_STAGE + (((4 * s4 + kb) ^ r) & 15) * 4);
+      const f32x4v a = *reinterpret_cast<const f32x4v*>(a_row + at + s4 * 16);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  int stage = 0;
+  for (; stage + 6 <= stages; stage += 3) {                 // every stage here has a successor three ahead
+    pass(w0); request(w0, stage + 3); multiply(stage);
+    pass(w1); request(w1, stage + 4); multiply(stage + 1);
+    pass(w2); request(w2, stage + 5); multiply(stage + 2);
+  }
+  const int left = stages - stage;                          // the last three to five stages: requests run out
+  pass(w0); if (left > 3) request(w0, stage + 3); multiply(stage);
+  pass(w1); if (left > 4) request(w1, stage + 4); multiply(stage + 1);
+  pass(w2); multiply(stage + 2);
+  if (left > 3) { pass(w0); multiply(stage + 3); }
+  if (left > 4) { pass(w1); multiply(stage + 4); }
+  float* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = 4 * kb + i, n = n0 + r;
+    if (m < M && n < N) out[(size_t)m * N + n] = acc[i];
+  }
+}
+
+static size_t fl_lds_bytes(int M, int K, int splits) {
+  return ((size_t)(M <= 8 ? 8 : 16) * (K / splits + FL_PAD) + (size_t)FL_WAVES * 16 * FL_STAGE) * sizeof(float);
+}
+
+static bool fl_takes(int M, int N, int K, int splits) {
+  return M >= 1 && M <= 16 && N >= 1 && splits >= 1 && K % (FL_STAGE * splits) == 0 &&
+         K / (FL_STAGE * splits) >= FL_DEPTH && fl_lds_bytes(M, K, splits) <= FL_LDS_LIMIT;
+}
+
+// The split of K for the whole-line kernel (0: it does not take the product): of the splits it takes (up to
+// 32), the one whose blocks fill their rounds of 256 CUs best, less 1.5 % a split for what the consumer of the
+// partial sums reads; one round of 160 blocks or more counts as full (the rule of the bfloat16 kernel).
+static int fl_splits(int M, int N, int K) {
+  const long column_blocks = (N + 16 * FL_WAVES - 1) / (16 * FL_WAVES);
+  int fit = 0;
+  double fit_score = 0;
+  for (int c = 1; c <= 32; ++c) {
+    if (!fl_takes(M, N, K, c)) continue;
+    const long blocks = column_blocks * c;
+    const long slots = blocks >= 160 && blocks <= 256 ? blocks : (blocks + 255) / 256 * 256;
+    const double score = (double)blocks / (double)slots - 0.015 * c;
+    if (!fit || score > fit_score) { fit = c; fit_score = score; }
+  }
+  return fit;
+}
+
 // Ways the few-row product will be split over K when partial sums are allowed (1: it is not split).
 extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
   if (M > SF_MOST_ROWS || K % 4) return 1;
+  if (const int lines = fl_splits(M, N, K)) return lines;
   const int column_blocks = (N + 127) / 128, steps = (K + 15) / 16;
   int sp = (768 + column_blocks - 1) / column_blocks;
   if (sp > 8) sp = 8;
@@ -196,6 +323,18 @@ extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, f
   if (K < 1 || splits < 1) return -1;
   const bool stream_ok = M <= SF_MOST_ROWS && K % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
   if (splits > 1 && (!stream_ok || bias)) return -1;
+  if (stream_ok && !bias && splits == fl_splits(M, N, K) && fl_takes(M, N, K, splits)) {
+    const size_t lds = fl_lds_bytes(M, K, splits);
+    static size_t granted = 0;
+    if (lds > 64 * 1024 && lds > granted) {
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_f32_lines_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+      granted = lds;
+    }
+    dim3 grid((N + 16 * FL_WAVES - 1) / (16 * FL_WAVES), 1, splits);
+    hipLaunchKernelGGL(gemm_f32_lines_kernel, grid, dim3(FL_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   if (stream_ok) {
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;           // 16-row tiles of A a block keeps
     const int steps = (K + 15) / 16, steps_per_split = (steps + splits - 1) / splits;

@@ -107,6 +107,24 @@ def test_linear_float32(ops, m, n, k, bias):
     check(ops.linear(x, w, b), want, torch.float32, scale=4)
 
 
+@pytest.mark.parametrize('k', [192, 256, 320, 384, 448, 512, 576, 1024, 4096])
+@pytest.mark.parametrize('m', [1, 8, 9, 16])
+def test_linear_float32_whole_lines(ops, m, k):
+    """The float32 product of up to 16 rows that reads W in whole cache lines: every number of stages from 3
+    on (the last three to five run apart from the inner ones), rows of W past the end of a wave's sixteen and
+    of a block's 128, whole and split over K; and a row's result does not depend on the rows beside it."""
+    n = 130 if k != 1024 else 2100
+    x, w = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5)
+    want = x.double() @ w.double().t()
+    assert ops.library.load().qil_gemm_f32_splits(m, n, k) >= 1
+    check(ops.linear(x, w, None), want, torch.float32, scale=4)
+    got = ops.linear(x, w, None, partials=True)
+    check(got.sum() if isinstance(got, ops.Partials) else got, want, torch.float32, scale=4)
+    alone = ops.linear(x[m - 1:].contiguous(), w, None, partials=True)
+    if isinstance(alone, ops.Partials) and isinstance(got, ops.Partials) and alone.splits == got.splits:
+        torch.testing.assert_close(alone.tensor[:, 0], got.tensor[:, m - 1], atol=0, rtol=0)
+
+
 @pytest.mark.parametrize('m,n,k', [(3, 1024, 4096), (16, 300, 2048), (20, 4096, 4096), (64, 1024, 3072), (33, 130, 516),
                                    (48, 2000, 100), (65, 512, 1024)])
 def test_linear_float32_partial_sums(ops, m, n, k):
