@@ -24,8 +24,10 @@ STREAM_GEMM_MAX_ROWS = 16
 # (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
 # the library says which products it takes (those of few column tiles).
 STREAM_GEMM_MOST_ROWS = 128
-# Keys per split of the row attention kernel.
+# Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
 ATTENTION_PART = 256
+# Blocks the row attention kernel aims for.
+ROWS_BLOCKS = 512
 # Blocks the matrix-core decode kernel aims for (256 CUs, 8 waves a block; measured best at 8 rows x 2048 keys).
 DECODE_BLOCKS = 256
 # Waves of a block of that kernel; each takes every DECODE_WAVES-th 32-key step of the block's keys.
@@ -311,6 +313,19 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
     return q
 
 
+def _rows_part(rows, kv_heads, max_context):
+    """Keys a part of the row kernel: about ROWS_BLOCKS blocks in all, parts of 64 to ATTENTION_PART * 2 keys
+    (measured in float32 at 2,048 keys of 8 kv heads: 1 row 36 us with parts of 64 against 54 with 256; 8 rows
+    best at 256; 64 rows best at 512)."""
+    if ATTENTION_PART != 256:                          # a test or tuning run has set it
+        return ATTENTION_PART
+    wanted = max_context * rows * kv_heads / ROWS_BLOCKS
+    part = 64
+    while part < 2 * ATTENTION_PART and part * 1.41 < wanted:      # the nearest of 64, 128, 256, 512
+        part *= 2
+    return part
+
+
 def _decode_parts(rows, kv_heads, max_context):
     """(keys a part, parts) of the matrix-core decode kernel: the context is split until the chip has enough blocks."""
     wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
@@ -463,7 +478,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), _ptr(single_rows), _ptr(out), rows, heads,
                                       head_dim, window_arg, part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:
-            part = ATTENTION_PART
+            part = _rows_part(rows, kv_heads, max_context)
             parts = max(1, -(-max_context // part))
             nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
             workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
