@@ -588,22 +588,26 @@ REAL = {
 }
 
 
-def test_twenty_requests_decode_together_at_real_sizes(tmp_path):
-    """Twenty requests through the serving loop at Qwen3-0.6B layer sizes in bfloat16: their decode steps have 17 to
-    64 rows (the products of that many rows, the attention kernel that does not make its own queries, a graph
-    of that batch size); every token is the plain sampler's choice on the plain logits, up to bfloat16's margin."""
+@pytest.mark.parametrize('count', [20, 100])
+def test_many_requests_decode_together_at_real_sizes(tmp_path, count):
+    """Twenty or a hundred requests through the serving loop at Qwen3-0.6B layer sizes in bfloat16: their decode
+    steps have 17 to 64 or 65 to 128 rows (the products of that many rows, the attention kernel that does not make
+    its own queries, a graph of that batch size); every token is the plain sampler's choice on the plain logits,
+    up to bfloat16's margin."""
     from qil_amd import Engine, Qwen3
     from conftest import write_model_folder
     config = REAL['0.6B']
     weights = plain.random_weights(config, 21)
     folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
     model = Qwen3.from_directory(folder, device='cuda', dtype=torch.bfloat16)
-    prompts = prompts_for(config, [3 + (7 * i) % 11 for i in range(20)], 9)
-    engine = Engine(model, num_pages=64, page_size=16, token_budget=256, prefill_chunk=64, max_active=20)
+    prompts = prompts_for(config, [3 + (7 * i) % 11 for i in range(count)], 9)
+    pages = 3 * count + 4
+    engine = Engine(model, num_pages=pages, page_size=16, token_budget=12 * count + 16, prefill_chunk=64, max_active=count)
     results = engine.generate(prompts, max_new_tokens=5, ignore_eos=True)
     assert engine.runner.graphs is None or engine.runner.graphs.replays >= 3
+    assert engine.runner.steps <= 8, 'the requests decode together'
     engine.cache.check()
-    assert engine.cache.free_pages == [64]
+    assert engine.cache.free_pages == [pages]
     # the margin in units of this model's logits (largest about 3.4, the tiny models' about 1)
     for prompt, result in zip(prompts, results):
         assert result['state'] == 'completed' and len(result['token_ids']) == 5
