@@ -2,7 +2,7 @@
 //   C[M, N] = A[M, K] W[N, K]^T (+ bias[N]),  float32 accumulation.
 // Four kernels, all bound by reading W once: `stream` (this comment; any shape, bias, unaligned operands),
 // `lines` (up to 16 rows, W in whole cache lines, optional merge of attention parts into A), `chunks`
-// (17 to 128 rows, A through LDS in stages) and `gated` (gate and up products with SiLU in the epilogue).
+// (17 to 192 rows, A through LDS in stages) and `gated` (gate and up products with SiLU in the epilogue).
 // Both operands have K contiguous (qil/model.py:32-40).  The product is bound by streaming W once
 // from HBM; A is small and would be re-read from L2 by every block, so the work is cut into wide,
 // short pieces: a block owns 128 * NT rows of W (8 waves, each 16 * NT rows) and ONE of `splits`
@@ -345,15 +345,15 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// The whole-line product for 17 to 128 rows of A and any length of K.  A does not stay in LDS as a whole
+// The whole-line product for 17 to 192 rows of A and any length of K.  A does not stay in LDS as a whole
 // slice: it passes through it one stage (128 columns) at a time, in two slots that the block's threads
 // fill in turn, from registers that are loaded three stages ahead, as W's are.  One barrier a stage: the
 // stage's slot has been written before it and the other slot may be written after it.  All waves of a
 // block are at the same stage, so the walk through K starts at a column of the block's (not the wave's) own.
 // MT: 16-row tiles of A (M <= 16 MT); every W fragment read from the buffer serves MT products.
-// Takes 16 < M <= 128, K a multiple of 128 per split with at least 3 stages, 16-byte aligned operands, no bias.
+// Takes 16 < M <= 192, K a multiple of 128 per split with at least 3 stages, 16-byte aligned operands, no bias.
 #define CHUNK_ROW (128 + GEMM_LDS_PAD)
-#define CHUNKS_MOST_ROWS 128
+#define CHUNKS_MOST_ROWS 192
 
 template <typename OUT, int MT>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
@@ -505,7 +505,9 @@ static int launch_chunks(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N,
   if (M <= 32) return launch_chunks_tiles<OUT, 2>(A, W, C, M, N, K, splits, s);
   if (M <= 64) return launch_chunks_tiles<OUT, 4>(A, W, C, M, N, K, splits, s);
   if (M <= 96) return launch_chunks_tiles<OUT, 6>(A, W, C, M, N, K, splits, s);
-  return launch_chunks_tiles<OUT, 8>(A, W, C, M, N, K, splits, s);
+  if (M <= 128) return launch_chunks_tiles<OUT, 8>(A, W, C, M, N, K, splits, s);
+  if (M <= 160) return launch_chunks_tiles<OUT, 10>(A, W, C, M, N, K, splits, s);
+  return launch_chunks_tiles<OUT, 12>(A, W, C, M, N, K, splits, s);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -780,14 +782,17 @@ extern "C" int qil_gemm_bf16_splits(int M, int N, int K) {
   return splits;
 }
 
-// 1 if a product with 17 to 128 rows should run on the weight-streaming kernel here (K a multiple of 128 of at
+// 1 if a product with 17 to 192 rows should run on the weight-streaming kernel here (K a multiple of 128 of at
 // least 384, no bias; operands 16-byte aligned, which the call checks); products of up to 16 rows always do.
 // 65 to 128 rows: only products of at most 64 column tiles (N <= 8192), which the split over K spreads over
 // the CUs; measured at 128 rows and 8B layer sizes against the GPU BLAS: 21 us against 26 (q/k/v), 16 against
 // 24 (attention output), 33 against 67 (down), but 57 against 49 for the 192 tiles of gate/up.
+// 129 to 192 rows (a portion of 128 tokens beside decoded ones): at most 32 column tiles; at 160 rows 19 against
+// 24 (attention output) and 39 against 60 (down), and level for the 48 tiles of q/k/v.
 extern "C" int qil_gemm_bf16_streams(int M, int N, int K, int has_bias) {
   if (M <= 16) return 1;
   if (M > 64 && N > 64 * 16 * LINES_WAVES) return 0;
+  if (M > 128 && N > 32 * 16 * LINES_WAVES) return 0;
   return chunks_takes(nullptr, nullptr, has_bias ? (const float*)1 : nullptr, M, N, K, 1);
 }
 

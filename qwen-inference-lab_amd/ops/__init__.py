@@ -22,8 +22,8 @@ STREAM_GEMM_MAX_ROWS = 16
 # ... and up to this many rows where K is a multiple of 128 (at least 384) and there is no bias: the kernel that
 # passes A through LDS in stages.  Measured at 64 rows and 8B layer sizes against the GPU BLAS: 41 us against 47
 # (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
-# the library says which products it takes (those of few column tiles).
-STREAM_GEMM_MOST_ROWS = 128
+# the library says which products it takes (those of few column tiles), and of 129 to 192 rows.
+STREAM_GEMM_MOST_ROWS = 192
 # Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
 ATTENTION_PART = 256
 # Blocks the row attention kernel aims for.

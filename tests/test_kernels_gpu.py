@@ -177,8 +177,8 @@ def test_linear_partial_sums(ops, m, n, k):
 
 
 @pytest.mark.parametrize('k', [384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 2432])
-@pytest.mark.parametrize('m', [17, 32, 33, 64, 65, 96, 97, 128])
-def test_linear_17_to_128_rows(ops, m, k):
+@pytest.mark.parametrize('m', [17, 32, 33, 64, 65, 96, 97, 128, 129, 160, 161, 192])
+def test_linear_17_to_192_rows(ops, m, k):
     """The kernel that passes A through LDS in stages, at every number of stages from 3 on (the first and the
     last stages run apart from the inner ones), at both numbers of row tiles, with rows of W past the end
     of a wave's and of a block's sixteen, whole and split over K."""
