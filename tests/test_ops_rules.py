@@ -1,0 +1,26 @@
+"""The host-side rules that choose how the attention kernels cut a context (no GPU needed)."""
+from qil_amd import ops
+
+
+def test_row_kernel_parts_scale_with_the_work():
+    """One row of 2,048 keys is cut into parts of 64 keys, eight rows into parts of 256, sixty-four into parts of
+    512; never below 64 or above 512, and a power of two."""
+    kv_heads = 8
+    assert ops._rows_part(1, kv_heads, 2048) == 64
+    assert ops._rows_part(8, kv_heads, 2048) == 256
+    assert ops._rows_part(8, kv_heads, 2100) == 256
+    assert ops._rows_part(64, kv_heads, 2048) == 512
+    assert ops._rows_part(1, 1, 5) == 64
+    assert ops._rows_part(128, 8, 100000) == 512
+    last = 0
+    for context in range(1, 40000, 977):
+        part = ops._rows_part(4, 2, context)
+        assert part in (64, 128, 256, 512) and part >= last
+        last = part
+
+
+def test_decode_parts_cover_the_context():
+    for rows, kv_heads, context in ((1, 8, 2048), (8, 8, 2048), (64, 8, 2048), (3, 1, 70000), (16, 4, 17), (1, 2, 1)):
+        part, parts = ops._decode_parts(rows, kv_heads, context)
+        assert part % 64 == 0 and ops.DECODE_MIN_PART <= part <= ops.DECODE_MAX_PART
+        assert parts >= 1 and part * parts >= context and part * (parts - 1) < context
