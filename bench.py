@@ -65,9 +65,11 @@ def main():
     parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
     parser.add_argument('--points', default='1,64', help='other decode batch sizes to report, comma separated')
     parser.add_argument('--prefill-tokens', type=int, default=2048)
-    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill', 'e2e'],
+    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill', 'e2e', 'mixed'],
                         help='measure only one phase (for profiling); the JSON line then lacks the other.  e2e: the '
-                             'reference\'s own workloads (output tokens over the wall time of whole requests)')
+                             'reference\'s own workloads (output tokens over the wall time of whole requests).  '
+                             'mixed: steps of one prompt portion (--portion tokens) beside --batch decoded rows')
+    parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')
     args = parser.parse_args()
     if args.gpus != 1:
         print(f'bench.py measures one GPU: this engine runs on a single MI355X (asked for {args.gpus})')
@@ -165,6 +167,33 @@ def main():
                 table[f'{length}x{count}'] = round(32 * count / statistics.median(times[1:]), 1)
         print(json.dumps({'e2e_output_tokens_per_s': table, 'sizes': NAMES[args.sizes], 'layers': args.layers,
                           'dtype': args.dtype}))
+        return 0
+    if args.phase == 'mixed':
+        # One request's prompt arrives in portions while `batch` others decode: every step is one batch of
+        # portion + batch rows, the decoding requests at --history tokens, the prompt growing from --history on.
+        steps = min(args.steps, 12)
+        room = args.history + steps * args.portion + 16
+        config_room = config['max_position_embeddings']
+        if room > config_room:
+            raise SystemExit(f'--history {args.history} and {steps} portions of {args.portion} need {room} positions, the model has {config_room}')
+        runner = ModelRunner(model, num_pages=(args.batch + 1) * (-(-room // page_size) + 1), page_size=page_size,
+                             max_requests=args.batch + 1)
+        for request in range(args.batch + 1):
+            runner.admit(request)
+            runner.step([StepEntry(request, tuple(prompt(args.history)), ())])
+        feed, times = prompt(room), []
+        for index in range(steps + 1):
+            entries = [StepEntry(args.batch, tuple(feed[index * args.portion:(index + 1) * args.portion]), (args.portion - 1,))]
+            entries += [StepEntry(request, (feed[request + index],), (0,)) for request in range(args.batch)]
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            logits = runner.step(entries)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - started)
+            assert logits.shape[0] == args.batch + 1 and torch.isfinite(logits).all()
+        print(json.dumps({'mixed_ms_per_step': round(statistics.median(times[1:]) * 1e3, 3), 'portion': args.portion,
+                          'decoded_rows': args.batch, 'history': args.history, 'layers': args.layers,
+                          'sizes': NAMES[args.sizes], 'dtype': args.dtype}))
         return 0
     if args.phase == 'prefill':
         prefill_s = prefill_run(args.prefill_tokens)

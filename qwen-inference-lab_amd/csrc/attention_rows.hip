@@ -181,26 +181,61 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
   }
 }
 
+// One wave a block; a head takes tg lanes (a power of two >= d / 4, four elements a lane), 64 / tg heads a wave.
+// The parts are read four at a time with all their loads first; the sums run over the parts in order.
 template <typename T>
-__global__ void attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
-                                       const float* __restrict__ part_l, const int* __restrict__ positions,
-                                       const int* __restrict__ row_index, T* __restrict__ out, int heads, int d,
-                                       int window, int P, int parts) {
-  const int slot_row = blockIdx.x, head = blockIdx.y;
+__global__ void __launch_bounds__(QIL_WAVE)
+attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
+                       const float* __restrict__ part_l, const int* __restrict__ positions,
+                       const int* __restrict__ row_index, T* __restrict__ out, int heads, int d,
+                       int window, int P, int parts, int tg) {
+  const int slot_row = blockIdx.x;
+  const int head = blockIdx.y * (QIL_WAVE / tg) + threadIdx.x / tg, e = (threadIdx.x % tg) * 4;
+  if (head >= heads || e >= d) return;
   const int row = row_index ? row_index[slot_row] : slot_row;
   const int ctx = positions[row] + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
   const int first = lo / P, last = (ctx - 1) / P;
   const size_t cell0 = ((size_t)slot_row * heads + head) * parts;
   float m = -INFINITY;
-  for (int p = first; p <= last; ++p) m = fmaxf(m, part_m[cell0 + p]);
-  float denom = 0.f;
-  for (int p = first; p <= last; ++p) denom += part_l[cell0 + p] * expf(part_m[cell0 + p] - m);
-  for (int e = threadIdx.x; e < d; e += blockDim.x) {
-    float numer = 0.f;
-    for (int p = first; p <= last; ++p) numer += part_acc[(cell0 + p) * d + e] * expf(part_m[cell0 + p] - m);
-    st(out + ((size_t)row * heads + head) * d + e, numer / denom);
+  for (int p0 = first; p0 <= last; p0 += 4) {
+    float mv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mv[j] = part_m[cell0 + min(p0 + j, last)];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, mv[j]);
   }
+  float denom = 0.f;
+  float4 numer = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int p0 = first; p0 <= last; p0 += 4) {
+    float mv[4], lv[4];
+    float4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const size_t cell = cell0 + min(p0 + j, last);
+      mv[j] = part_m[cell];
+      lv[j] = part_l[cell];
+      acc[j] = *reinterpret_cast<const float4*>(part_acc + cell * d + e);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (p0 + j <= last) {
+        const float f = expf(mv[j] - m);
+        denom += lv[j] * f;
+        numer.x += acc[j].x * f; numer.y += acc[j].y * f; numer.z += acc[j].z * f; numer.w += acc[j].w * f;
+      }
+    }
+  }
+  T* to = out + ((size_t)row * heads + head) * d + e;
+  st(to, numer.x / denom); st(to + 1, numer.y / denom); st(to + 2, numer.z / denom); st(to + 3, numer.w / denom);
+}
+
+// Launch shape of the merge: lanes a head and the grid.
+static void merge_shape(int rows, int heads, int d, int* tg, dim3* grid) {
+  int lanes = 1;
+  while (lanes * 4 < d) lanes *= 2;
+  *tg = lanes;                                             // d <= 256: at most 64
+  *grid = dim3(rows, (heads + QIL_WAVE / lanes - 1) / (QIL_WAVE / lanes));
 }
 
 static int next_pow2_log2(int v) {
@@ -237,8 +272,11 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
 #undef QIL_ROWS_CASE
   int status = (int)hipGetLastError();
   if (status || parts == 1) return status;
-  hipLaunchKernelGGL(attn_rows_merge_kernel<T>, dim3(rows, heads), dim3(d >= 128 ? 128 : 64), 0, s, part_acc, part_m,
-                     part_l, positions, row_index, (T*)out, heads, d, window, P, parts);
+  int tg;
+  dim3 merge_grid;
+  merge_shape(rows, heads, d, &tg, &merge_grid);
+  hipLaunchKernelGGL(attn_rows_merge_kernel<T>, merge_grid, dim3(QIL_WAVE), 0, s, part_acc, part_m, part_l, positions,
+                     row_index, (T*)out, heads, d, window, P, parts, tg);
   return (int)hipGetLastError();
 }
 
@@ -281,13 +319,17 @@ int qil_attn_merge(const void* workspace, const int* positions, const int* row_i
   const float* acc = (const float*)workspace;
   const float* m = acc + (size_t)rows * heads * parts * d;
   const float* l = m + (size_t)rows * heads * parts;
-  const dim3 grid(rows, heads), block(d >= 128 ? 128 : 64);
+  if (d % 4 || d > 256) return -1;
+  int tg;
+  dim3 grid;
+  merge_shape(rows, heads, d, &tg, &grid);
+  const dim3 block(QIL_WAVE);
   if (dtype == QIL_F32)
     hipLaunchKernelGGL(attn_rows_merge_kernel<float>, grid, block, 0, s, acc, m, l, positions, row_index, (float*)out,
-                       heads, d, window, P, parts);
+                       heads, d, window, P, parts, tg);
   else
     hipLaunchKernelGGL(attn_rows_merge_kernel<bf16_t>, grid, block, 0, s, acc, m, l, positions, row_index, (bf16_t*)out,
-                       heads, d, window, P, parts);
+                       heads, d, window, P, parts, tg);
   QIL_RETURN_LAUNCH_STATUS();
 }
 
