@@ -12,6 +12,12 @@ bucket's end.
 With a sampler the draw of the next tokens is part of the graph too (its seeds, output indices and
 temperatures travel in the same array), and a step costs one upload, one replay and one download.
 
+Steps with prompt portions have recurring shapes too (a portion of the chunk size beside so many single
+tokens, step after step while a long prompt comes in), and for small models their launches cost more than
+their kernels.  A shape that has been seen before (the same numbers of tokens and of wanted places per request,
+largest first, and the same, wider bucket) is captured the second time and replayed from then on; the
+requests are put into the graph's order and the logits back into the caller's.  The draw stays outside.
+
 Nothing in the captured region clears memory with a memset node: buffers are allocated, not
 zeroed, and kernels write every element they later read.
 """
@@ -25,6 +31,10 @@ from .batch import StepEntry
 
 BUCKET = 512          # contexts are rounded up to a multiple of this many tokens for a graph
 MAX_GRAPHS = 12
+MIXED_BUCKET = 2048   # ... and of this many for a step with prompt portions (a portion moves on by its size a step)
+MIXED_MOST_ROWS = 512  # steps of more rows are bound by their kernels, not by their launches
+MAX_MIXED_GRAPHS = 8
+MAX_SEEN = 256        # shapes remembered as seen once
 
 
 class _Graph:
@@ -135,13 +145,70 @@ class DecodeGraphs:
     def __init__(self, runner):
         self._runner, self.graphs, self.replays, self.captures = weakref.ref(runner), {}, 0, 0     # no cycle
         self._safe = None
+        self.mixed, self.seen, self.mixed_replays, self.mixed_captures = {}, {}, 0, 0
 
-    def takes(self, entries):
+    def safe(self):
         if self._safe is None:
             blocks = self._runner().model.blocks
             self._safe = all(b.mixer is None or b.mixer.graph_safe for b in blocks)
-        return self._safe and all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
+        return self._safe
+
+    def takes(self, entries):
+        return self.safe() and all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
                    tuple(e[2] if not isinstance(e, StepEntry) else e.want) == (0,) for e in entries) and len(entries) > 0
+
+    def mixed_step(self, entries):
+        """(logits, entries, starts) of a step with prompt portions from a graph of its shape, or None: the shape
+        is new (it is remembered), too large, or a mixer reads the host side of the step."""
+        if not self.safe() or not entries:
+            return None
+        runner = self._runner()
+        normal = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2]) if len(e) > 2 else ())
+                  for e in entries]
+        if sum(len(e.tokens) for e in normal) > MIXED_MOST_ROWS or max(len(e.tokens) for e in normal) < 2:
+            return None
+        runner._validate(normal)
+        # the graph's order: most tokens first, the caller's order among equals
+        order = sorted(range(len(normal)), key=lambda i: (-len(normal[i].tokens), -len(normal[i].want), i))
+        ordered = [normal[i] for i in order]
+        ps = runner.cache.page_size
+        longest = max(runner.cache.computed[e.request] + len(e.tokens) for e in ordered)
+        bucket = -(-longest // MIXED_BUCKET) * MIXED_BUCKET
+        limit = runner.max_positions
+        if limit is not None:
+            bucket = min(bucket, -(-limit // ps) * ps)
+        width = -(-bucket // ps)
+        key = (tuple(len(e.tokens) for e in ordered), tuple(len(e.want) for e in ordered), bucket)
+        graph = self.mixed.get(key)
+        if graph is None:
+            if key not in self.seen:                       # a shape's first time: run it launch by launch
+                if len(self.seen) >= MAX_SEEN:
+                    self.seen.clear()
+                self.seen[key] = True
+                return None
+            if len(self.mixed) >= MAX_MIXED_GRAPHS:
+                self.mixed.pop(next(iter(self.mixed)))
+            described, pieces, facts = runner._describe(ordered, table_width=width, validate=False)
+            graph = self.mixed[key] = _Graph(runner, described, pieces, facts, bucket)
+            self.mixed_captures += 1
+        else:
+            described, pieces, facts = runner._describe(ordered, table_width=width, validate=False)
+            graph.load(pieces)
+        logits = graph.run()
+        self.mixed_replays += 1
+        if logits is not None:
+            # rows of the wanted places in the caller's order of requests
+            first, at = {}, 0
+            for index, entry in zip(order, ordered):
+                first[index] = at
+                at += len(entry.want)
+            back = [first[i] + j for i in range(len(normal)) for j in range(len(normal[i].want))]
+            if back != list(range(len(back))):
+                logits = logits.index_select(0, torch.tensor(back, dtype=torch.int64).to(logits.device, non_blocking=True))
+            else:
+                logits = logits.clone()                     # the graph's own output buffer is overwritten by the next replay
+        starts = {e.request: s for e, s in zip(ordered, facts['starts'])}
+        return logits, normal, [starts[e.request] for e in normal]
 
     def step(self, entries, sampler=None, packed=None):
         """(logits, entries, starts) of a decode batch; with a sampler and its packed parameters the first

@@ -140,13 +140,21 @@ class ModelRunner:
         if self.graphs is not None and self.graphs.takes(entries):
             logits, entries, starts = self.graphs.step(entries)
         else:
-            entries, ctx = self.prepare(entries)
-            logits = self.model.forward(ctx, self.views)
-            starts = ctx.host_starts
+            logits, entries, starts = self._forward(entries)
         for entry, start in zip(entries, starts):
             self.cache.advance(entry.request, start + len(entry.tokens))
         self.steps += 1
         return logits
+
+    def _forward(self, entries):
+        """(logits, entries, starts) of a step that is no decode batch: from a graph of its shape if there is
+        one, else launch by launch."""
+        if self.graphs is not None:
+            replayed = self.graphs.mixed_step(entries)
+            if replayed is not None:
+                return replayed
+        entries, ctx = self.prepare(entries)
+        return self.model.forward(ctx, self.views), entries, ctx.host_starts
 
     @torch.inference_mode()
     def step_and_sample(self, entries, sampler, params, counters):
@@ -157,9 +165,7 @@ class ModelRunner:
         if self.graphs is not None and self.graphs.takes(entries):
             drawn, entries, starts = self.graphs.step(entries, sampler, packed)
         else:
-            entries, ctx = self.prepare(entries)
-            logits = self.model.forward(ctx, self.views)
-            starts = ctx.host_starts
+            logits, entries, starts = self._forward(entries)
             drawn = None
             if logits is not None:
                 if logits.shape[0] != packed.shape[1]:

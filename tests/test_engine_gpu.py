@@ -618,6 +618,48 @@ def test_many_requests_decode_together_at_real_sizes(tmp_path, count):
     engine.close()
 
 
+def test_portions_of_a_long_prompt_replay_a_graph_at_real_sizes(tmp_path):
+    """A 128-token portion beside three decoded rows at Qwen3-0.6B layer sizes, eight steps: the library's
+    products (gate/up at 131 rows) and this repository's kernels inside a replayed graph, every replay against
+    a runner without graphs and against the plain model."""
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.weights import load_model
+    from conftest import write_model_folder
+    config = REAL['0.6B']
+    weights = plain.random_weights(config, 11)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    model = load_model(folder, dtype=torch.bfloat16, device='cuda')
+    prompts = dict(zip('pabc', prompts_for(config, [1100, 90, 40, 300], 5)))
+    outputs = []
+    for flag in (True, False):
+        runner = ModelRunner(model, num_pages=120, page_size=16, max_requests=4, graphs=flag)
+        for group in runner.cache.kv_groups:
+            group['k'].fill_(float('nan')), group['v'].fill_(float('nan'))
+        fed = {}
+        for r, head in (('p', 70), ('a', 80), ('b', 30), ('c', 290)):
+            runner.admit(r)
+            runner.step([StepEntry(r, tuple(prompts[r][:head]), ())])
+            fed[r] = head
+        rows = []
+        for turn in range(8):
+            entries = [StepEntry(r, tuple(prompts[r][fed[r]:fed[r] + (128 if r == 'p' else 1)]), (127,) if r == 'p' else (0,))
+                       for r in ('abcp' if turn % 2 else 'pcba')]
+            logits = runner.step(entries).cpu()
+            for index, entry in enumerate(entries):
+                fed[entry.request] += len(entry.tokens)
+                rows.append((entry.request, fed[entry.request] - 1, logits[index]))
+            torch.cuda.synchronize()
+        if flag:
+            assert runner.graphs.mixed_captures == 1 and runner.graphs.mixed_replays == 7
+        outputs.append(rows)
+    expected = {r: plain.logits(prompts[r][:fed[r]], weights, config) for r in prompts}
+    for (r, place, with_graph), (_, _, eager) in zip(*outputs):
+        scale = max(1.0, expected[r].abs().max().item())
+        assert torch.isfinite(with_graph).all()
+        torch.testing.assert_close(with_graph, eager, atol=0.008 * scale, rtol=0.02)
+        torch.testing.assert_close(with_graph, expected[r][place], atol=0.015 * scale, rtol=0.02)
+
+
 @pytest.mark.parametrize('name,dtype', [('0.6B', torch.float32), ('0.6B', torch.bfloat16), ('8B', torch.bfloat16),
                                         ('4B', torch.bfloat16), ('14B', torch.bfloat16)])
 def test_layers_of_real_size(tmp_path, name, dtype):

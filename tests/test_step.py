@@ -239,6 +239,54 @@ def test_graph_replays_equal_eager_launches(model_folder, dtype):
     torch.testing.assert_close(got, expected[5:13], **TOLERANCE[dtype])
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_steps_with_portions_replay_a_graph_of_their_shape(model_folder, dtype):
+    """A shape of step that comes again (a portion of five tokens beside two decoded tokens, the requests in
+    another order every step) runs launch by launch the first time, is captured the second time and replayed
+    from then on, with other work between the replays; every step's logits are those of a runner without graphs
+    up to the order of sums in attention (the graph cuts the context by its bucket), and the plain model's."""
+    config, seed, page_size = CONFIGS['B']
+    folder, weights = model_folder(config, seed)
+    model = load_model(folder, dtype=dtype, device='cuda')
+    prompts = {r: tokens_for(config, n, 70 + n) for r, n in (('p', 60), ('a', 30), ('b', 30), ('other', 25))}
+    outputs = []
+    for flag in (True, False):
+        runner = ModelRunner(model, num_pages=40, page_size=page_size, graphs=flag)
+        poison(runner)
+        fed = {}
+        for r, head in (('p', 4), ('a', 9), ('b', 13), ('other', 2)):
+            runner.admit(r)
+            runner.step([StepEntry(r, tuple(prompts[r][:head]), ())])
+            fed[r] = head
+        got = {r: [] for r in 'pab'}
+        for turn in range(9):
+            order = ['p', 'a', 'b'] if turn % 3 == 0 else ['a', 'p', 'b'] if turn % 3 == 1 else ['b', 'a', 'p']
+            entries = [StepEntry(r, tuple(prompts[r][fed[r]:fed[r] + (5 if r == 'p' else 1)]), (4, 0) if r == 'p' else (0,))
+                       for r in order]
+            logits = runner.step(entries)
+            at = 0
+            for entry in entries:
+                for w in entry.want:
+                    got[entry.request].append((fed[entry.request] + w, logits[at].cpu()))
+                    at += 1
+                fed[entry.request] += len(entry.tokens)
+            runner.step([StepEntry('other', tuple(prompts['other'][fed['other']:fed['other'] + 2]), ())])   # other work in between
+            fed['other'] += 2
+            torch.cuda.synchronize()
+        if flag:
+            assert runner.graphs.mixed_captures == 2 and runner.graphs.mixed_replays >= 14, \
+                (runner.graphs.mixed_captures, runner.graphs.mixed_replays)      # the step's shape and the other work's
+        runner.cache.check()
+        outputs.append(got)
+    for r in 'pab':
+        expected = plain.logits(prompts[r], weights, config)
+        for (place, with_graph), (same_place, eager) in zip(outputs[0][r], outputs[1][r]):
+            assert place == same_place
+            torch.testing.assert_close(with_graph, eager, **TOLERANCE[dtype])
+            torch.testing.assert_close(with_graph, expected[place], **TOLERANCE[dtype])
+
+
 def random_configuration(r):
     """Every size and option drawn at random: head sizes in steps of 16 up to 256, one to eight kv heads with
     groups of one to sixteen, widths and vocabularies that are no powers of two, biases, tied or own head."""
