@@ -618,21 +618,23 @@ def test_many_requests_decode_together_at_real_sizes(tmp_path, count):
     engine.close()
 
 
-def test_portions_of_a_long_prompt_replay_a_graph_at_real_sizes(tmp_path):
-    """A 128-token portion beside three decoded rows at Qwen3-0.6B layer sizes, eight steps: the library's
-    products (gate/up at 131 rows) and this repository's kernels inside a replayed graph, every replay against
-    a runner without graphs and against the plain model."""
+@pytest.mark.parametrize('name,portions', [('0.6B', 1), ('0.6B', 4), ('8B', 4)])
+def test_portions_of_a_long_prompt_replay_a_graph_at_real_sizes(tmp_path, name, portions):
+    """A 128-token portion beside three decoded rows (131 rows), or four portions (512 rows: every product the
+    library's), at Qwen3-0.6B layer sizes, eight steps: the library's products and this repository's kernels
+    (or 8B: other kernels of the library) inside a replayed graph, every replay against a runner without graphs
+    and against the plain model."""
     from qil_amd.engine import ModelRunner, StepEntry
     from qil_amd.weights import load_model
     from conftest import write_model_folder
-    config = REAL['0.6B']
+    config = REAL[name]
     weights = plain.random_weights(config, 11)
     folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
     model = load_model(folder, dtype=torch.bfloat16, device='cuda')
-    prompts = dict(zip('pabc', prompts_for(config, [1100, 90, 40, 300], 5)))
+    prompts = dict(zip('pabc', prompts_for(config, [1100, 90, 40, 300] if portions == 1 else [1100, 1110, 1060, 1320], 5)))
     outputs = []
     for flag in (True, False):
-        runner = ModelRunner(model, num_pages=120, page_size=16, max_requests=4, graphs=flag)
+        runner = ModelRunner(model, num_pages=120 if portions == 1 else 300, page_size=16, max_requests=4, graphs=flag)
         for group in runner.cache.kv_groups:
             group['k'].fill_(float('nan')), group['v'].fill_(float('nan'))
         fed = {}
@@ -642,7 +644,8 @@ def test_portions_of_a_long_prompt_replay_a_graph_at_real_sizes(tmp_path):
             fed[r] = head
         rows = []
         for turn in range(8):
-            entries = [StepEntry(r, tuple(prompts[r][fed[r]:fed[r] + (128 if r == 'p' else 1)]), (127,) if r == 'p' else (0,))
+            long = 'p' if portions == 1 else 'pabc'
+            entries = [StepEntry(r, tuple(prompts[r][fed[r]:fed[r] + (128 if r in long else 1)]), (127,) if r in long else (0,))
                        for r in ('abcp' if turn % 2 else 'pcba')]
             logits = runner.step(entries).cpu()
             for index, entry in enumerate(entries):
