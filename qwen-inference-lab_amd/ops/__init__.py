@@ -38,8 +38,9 @@ DECODE_MIN_PART = 256
 DECODE_MAX_PART = 8192
 # Rows up to which a decode step makes its queries, new keys and values inside the attention kernel: with few
 # rows that saves a launch; with many the kernel is bound by memory and the blocks' start costs more than the
-# launch (64 rows of 2048 keys: 111 us against 94 + 5).
-FUSED_DECODE_MOST_ROWS = 16
+# launch (64 rows of 2048 keys: 111 us against 94 + 5; whole steps at 8B sizes: 24 and 32 rows gain 0.8 %
+# with the fused kernel, 48 rows lose 2 %).
+FUSED_DECODE_MOST_ROWS = 32
 # Launches of at most this many blocks (one a CU) let a wave load two of its steps at a time.
 DECODE_PAIRS_BLOCKS = 256
 

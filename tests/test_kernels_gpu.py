@@ -424,6 +424,7 @@ def test_linear_merges_unmerged_attention(ops, lengths, window, d, heads, kv_hea
     ([257, 512, 513], 32, 128, 8, 1, 100, False, 64, 1),                               # no norm, half of the head rotated, a window
     ([40, 1000], 16, 64, 16, 1, None, True, 0, 2),                                     # 16 heads a kv head, no rotation
     ([5000], 16, 128, 5, 5, None, True, 32, 5),                                        # one head a kv head, many parts
+    ([37 * i % 900 + 1 for i in range(30)], 16, 128, 16, 8, None, True, 128, 4),       # thirty rows
 ])
 def test_decode_attention_fused_is_the_two_kernels(ops, lengths, page_size, d, heads, kv_heads, window, norm, rot, splits):
     """Queries, new key and new value made inside the attention kernel from the q/k/v product's partial sums:
