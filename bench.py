@@ -106,8 +106,8 @@ def main():
                         prefill_chunk=args.history, max_active=batch)
         ids = [engine.submit(prompt(args.history), max_new_tokens=new_tokens, ignore_eos=True)
                for _ in range(batch)]
-        requests = engine.scheduler.requests
-        while any(requests[i].computed < args.history for i in ids):      # untimed: histories into the cache
+        computed = engine.scheduler.computed
+        while any(engine.result(i)['state'] == 'waiting' or computed(i) < args.history for i in ids):      # untimed: histories into the cache
             engine.step()
         for _ in range(args.warmup):
             engine.step()
@@ -119,7 +119,7 @@ def main():
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
         assert produced == batch * args.steps, 'a decode step must produce one token per request'
-        contexts = [requests[i].computed - args.steps // 2 for i in ids]
+        contexts = [computed(i) - args.steps // 2 for i in ids]
         engine.close()
         engine.cache.check()
         assert engine.cache.free_pages == [pages], 'pages leaked'

@@ -1,4 +1,4 @@
-"""python -m qil_amd --model DIR --token-ids '[1, 2, 3]' --dtype bfloat16
+"""qil-amd (or python -m qil_amd) --model DIR --token-ids '[1, 2, 3]' --dtype bfloat16
 
 Options and meanings follow the reference's command line (qil/__main__.py:8-21):
 --model, --prompt | --token-ids, --device, --dtype, --max-new-tokens, --pages,
@@ -9,11 +9,12 @@ write a random model folder into --model first.
 """
 import argparse
 import json
+import sys
 from pathlib import Path
 
 
-def main(argv=None):
-    parser = argparse.ArgumentParser(prog='python -m qil_amd', description=__doc__)
+def options():
+    parser = argparse.ArgumentParser(prog='qil-amd', description=__doc__)
     parser.add_argument('--model', required=True, help='model folder (config.json + *.safetensors)')
     source = parser.add_mutually_exclusive_group(required=True)
     source.add_argument('--prompt', help='text; needs tokenizer.json in the model folder')
@@ -32,40 +33,46 @@ def main(argv=None):
     parser.add_argument('--random-config', help='JSON file or string: write random weights for it into --model first')
     parser.add_argument('--random-seed', default=0, type=int)
     parser.add_argument('--output', type=Path)
-    args = parser.parse_args(argv)
+    return parser
 
+
+def prompt_tokens(args):
+    """(token ids, decoder of token ids to text or None) from --token-ids or --prompt."""
+    if args.token_ids is not None:
+        return json.loads(args.token_ids), None
+    from tokenizers import Tokenizer
+    tokenizer = Tokenizer.from_file(str(Path(args.model) / 'tokenizer.json'))
+    return (tokenizer.encode(args.prompt, add_special_tokens=False).ids,
+            lambda ids: tokenizer.decode(ids, skip_special_tokens=True))
+
+
+def main(argv=None):
+    args = options().parse_args(argv)
     import torch
     from .engine import Engine
     from .weights import load_model, write_random_model
-    dtype = getattr(torch, args.dtype)
     if args.random_config:
-        text = args.random_config
-        data = json.loads(Path(text).read_text() if not text.lstrip().startswith('{') else text)
-        write_random_model(args.model, data, args.random_seed)
-    tokenizer = None
-    if args.prompt is not None:
-        from tokenizers import Tokenizer
-        tokenizer = Tokenizer.from_file(str(Path(args.model) / 'tokenizer.json'))
-        tokens = tokenizer.encode(args.prompt, add_special_tokens=False).ids
-    else:
-        tokens = json.loads(args.token_ids)
-    model = load_model(args.model, dtype=dtype, device=args.device)
+        given = args.random_config
+        source = given if given.lstrip().startswith('{') else Path(given).read_text()
+        write_random_model(args.model, json.loads(source), args.random_seed)
+    tokens, to_text = prompt_tokens(args)
+    model = load_model(args.model, dtype=getattr(torch, args.dtype), device=args.device)
     engine = Engine(model, num_pages=args.pages, page_size=args.page_size, prefill_chunk=args.chunk_size,
                     token_budget=args.token_budget, max_active=args.max_active)
     try:
-        result = engine.generate([tokens], max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos,
-                                 temperature=args.temperature, seed=args.seed)[0]
-        if tokenizer is not None:
-            result['text'] = tokenizer.decode(result['token_ids'], skip_special_tokens=True)
-        encoded = json.dumps(result, ensure_ascii=False, indent=2)
-        if args.output:
-            args.output.parent.mkdir(parents=True, exist_ok=True)
-            args.output.write_text(encoded + '\n')
-        print(encoded)
+        report, = engine.generate([tokens], max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos,
+                                  temperature=args.temperature, seed=args.seed)
     finally:
         engine.close()
+    if to_text is not None:
+        report['text'] = to_text(report['token_ids'])
+    text = json.dumps(report, ensure_ascii=False, indent=2) + '\n'
+    sys.stdout.write(text)
+    if args.output is not None:
+        args.output.parent.mkdir(parents=True, exist_ok=True)
+        args.output.write_text(text)
     return 0
 
 
 if __name__ == '__main__':
-    raise SystemExit(main())
+    sys.exit(main())

@@ -1,23 +1,40 @@
-"""Round-robin planner with a token budget, chunked prompts and admission between steps.
+"""Which requests run in the next step, and with how many of their tokens.
 
-Policy of the reference's scheduler (qil/scheduler.py:37-103):
-  * ``add`` refuses a request that could never fit the cache (:52-53).
-  * ``plan`` first admits waiting requests while fewer than ``max_active`` are
-    active and the cache can reserve their whole life (``len(prompt) +
-    max_new_tokens - 1`` tokens: the last sampled token is never fed back,
-    :24-27); a request that does not fit goes to the back of the queue, so a
-    smaller later one may overtake it (:58-67).
-  * then it hands out the step's token budget: at most one piece of work per
-    active request, ``prefill_chunk`` tokens of a prompt or the one last sampled
-    token of a decoding request, cut down to the remaining budget; served
-    requests rotate to the back, so those left out come first next step (:68-84).
-  * pages cannot run out inside a request, because admission reserved them; lack
-    of room shows as waiting, or as refusal at ``add``.  Nothing is preempted,
-    swapped or recomputed.
-The plan is executed as one batch by the step function.
+The policy is the reference's (qil/scheduler.py:57-87), the bookkeeping is this engine's:
+
+  admission   between steps, while fewer than ``max_active`` requests run: the oldest waiting
+              request whose whole life (``len(prompt) + max_new_tokens - 1`` cached tokens; the last
+              drawn token is never fed back, qil/scheduler.py:24-27) the cache can reserve now.  One
+              that does not fit keeps waiting behind those not yet asked, so a smaller, later one may
+              overtake it.  One that could never fit is refused when it is added.
+  budget      a step holds at most ``token_budget`` tokens.  Running requests are served in turn, one
+              piece each: up to ``prefill_chunk`` tokens of a prompt, or the one token drawn last; the
+              piece is cut to what is left of the budget.  Requests that were served go behind those
+              that were not, so nobody starves at a budget of one.
+  progress    how far a request has come is the cache manager's count of its cached tokens; the
+              scheduler keeps no second counter.
+  pages       cannot run out inside a request (admission reserved them).  Nothing is preempted,
+              swapped or recomputed.
+
+A piece of work knows whether it ends at the request's last known token, i.e. whether the step has to
+draw a token for it; the step function's entry is made from it directly.
 """
-from collections import deque
+import enum
 from dataclasses import dataclass, field
+
+from .batch import StepEntry
+
+
+class Phase(enum.Enum):
+    WAITING = 'waiting'
+    ACTIVE = 'active'
+    COMPLETED = 'completed'
+    CANCELLED = 'cancelled'
+    FAILED = 'failed'
+
+    @property
+    def live(self):
+        return self in (Phase.WAITING, Phase.ACTIVE)
 
 
 @dataclass
@@ -31,89 +48,136 @@ class Request:
     seed: int = 0
     output: list = field(default_factory=list)
     token_times_s: list = field(default_factory=list)
-    computed: int = 0
-    state: str = 'waiting'               # waiting -> active -> completed | cancelled | failed
+    phase: Phase = Phase.WAITING
     finish_reason: str | None = None
     error: str | None = None
 
     @property
-    def input_tokens(self):
-        return self.prompt + self.output
+    def state(self):
+        return self.phase.value
+
+    @property
+    def known(self):
+        """Tokens that exist so far: the prompt and what was drawn."""
+        return len(self.prompt) + len(self.output)
 
     @property
     def cache_limit(self):
         return len(self.prompt) + self.max_new_tokens - 1
 
+    def span(self, lo, hi):
+        """Tokens lo..hi-1 of prompt + output, without joining the two lists (that copy grows with the context)."""
+        edge = len(self.prompt)
+        if hi <= edge:
+            return tuple(self.prompt[lo:hi])
+        if lo >= edge:
+            return tuple(self.output[lo - edge:hi - edge])
+        return tuple(self.prompt[lo:]) + tuple(self.output[:hi - edge])
+
+    def accept(self, token, now):
+        """Take a drawn token; the reason why the request is finished with it, or None."""
+        self.output.append(token)
+        self.token_times_s.append(now)
+        if token in self.eos:
+            return 'eos'
+        return 'length' if len(self.output) >= self.max_new_tokens else None
+
+    def report(self):
+        """The caller's view of the request (fields of qil/engine.py:120-131): times are since arrival."""
+        since = [t - self.arrival_s for t in self.token_times_s]
+        steps = len(since) - 1
+        return dict(request_id=self.id, state=self.state, finish_reason=self.finish_reason, error=self.error,
+                    token_ids=list(self.output), token_times_s=since,
+                    ttft_s=since[0] if since else None,
+                    e2e_s=since[-1] if self.phase is Phase.COMPLETED and since else None,
+                    tpot_s=(since[-1] - since[0]) / steps if steps > 0 else None)
+
 
 @dataclass(frozen=True)
 class Work:
+    """One request's share of a step."""
     request_id: int
-    start: int
+    start: int              # position of its first token = tokens cached before the step
     tokens: tuple
+    draws: bool             # the piece ends at the last known token: the step draws the next one
+
+    def entry(self):
+        return StepEntry(self.request_id, self.tokens, (len(self.tokens) - 1,) if self.draws else ())
 
 
 class Scheduler:
     def __init__(self, cache, *, token_budget=128, prefill_chunk=64, max_active=4):
-        if any(type(n) is not int or n < 1 for n in (token_budget, prefill_chunk, max_active)):
-            raise ValueError('scheduler budgets must be positive integers')
-        self.cache, self.token_budget, self.prefill_chunk, self.max_active = cache, token_budget, prefill_chunk, max_active
-        self.requests, self.waiting, self.active = {}, deque(), deque()
+        for name, value in (('token_budget', token_budget), ('prefill_chunk', prefill_chunk), ('max_active', max_active)):
+            if type(value) is not int or value < 1:
+                raise ValueError(f'{name} must be a positive integer, not {value!r}')
+        self.cache = cache
+        self.token_budget, self.prefill_chunk, self.max_active = token_budget, prefill_chunk, max_active
+        self.requests = {}
+        self.waiting, self.active = [], []          # request ids, oldest (or next to be served) first
 
+    # ------------------------------------------------------------------ arrivals and departures
     def add(self, request):
         if request.id in self.requests:
-            raise ValueError('duplicate request ID')
+            raise ValueError(f'duplicate request id {request.id!r}')
         if not self.cache.fits_at_all(request.cache_limit):
-            raise ValueError('request exceeds total KV capacity; reduce tokens or increase pages')
+            raise ValueError(f'a request of {request.cache_limit} cached tokens exceeds the cache\'s total capacity: '
+                             'fewer tokens or more pages')
         self.requests[request.id] = request
         self.waiting.append(request.id)
 
-    def plan(self):
-        for _ in range(len(self.waiting)):
-            if len(self.active) >= self.max_active:
-                break
-            request_id = self.waiting.popleft()
-            request = self.requests[request_id]
-            if self.cache.admit(request_id, request.cache_limit):
-                request.state = 'active'
-                self.active.append(request_id)
-            else:
-                self.waiting.append(request_id)
-        remaining, work = self.token_budget, []
-        for _ in range(len(self.active)):
-            if not remaining:
-                break
-            request_id = self.active.popleft()
-            request = self.requests[request_id]
-            at, prompt_length = request.computed, len(request.prompt)
-            chunk = self.prefill_chunk if at < prompt_length else 1
-            count = min(chunk, remaining, prompt_length + len(request.output) - at)
-            if count <= 0:
-                raise RuntimeError('active request has no input to compute')
-            if at + count <= prompt_length:           # slices, not prompt + output: that copy grows with the context
-                tokens = request.prompt[at:at + count]
-            elif at >= prompt_length:
-                tokens = request.output[at - prompt_length:at - prompt_length + count]
-            else:
-                tokens = request.prompt[at:] + request.output[:at + count - prompt_length]
-            work.append(Work(request_id, at, tuple(tokens)))
-            remaining -= count
-            self.active.append(request_id)
-        if not work and self.waiting:
-            raise RuntimeError('no runnable request despite an empty active set')
-        return work
-
-    def retire(self, request_id, state, reason):
+    def retire(self, request_id, phase, reason):
+        """Take a live request out (its pages go back); False if it was not live any more."""
         request = self.requests[request_id]
-        if request.state not in ('waiting', 'active'):
+        if not request.phase.live:
             return False
-        if request_id in self.waiting:
-            self.waiting.remove(request_id)
-        if request_id in self.active:
+        if request.phase is Phase.ACTIVE:
             self.active.remove(request_id)
             self.cache.release(request_id)
-        request.state, request.finish_reason = state, reason
+        else:
+            self.waiting.remove(request_id)
+        request.phase, request.finish_reason = Phase(phase), reason
         return True
+
+    def computed(self, request_id):
+        """Tokens of an active request that are in the cache."""
+        return self.cache.computed[request_id]
 
     @property
     def idle(self):
-        return not self.waiting and not self.active
+        return not (self.waiting or self.active)
+
+    # ------------------------------------------------------------------ the plan of one step
+    def _admit(self):
+        queue, passed_over = self.waiting, []
+        while queue and len(self.active) < self.max_active:
+            request = self.requests[queue.pop(0)]
+            if self.cache.admit(request.id, request.cache_limit):
+                request.phase = Phase.ACTIVE
+                self.active.append(request.id)
+            else:
+                passed_over.append(request.id)
+        self.waiting = queue + passed_over
+
+    def _share(self):
+        left, pieces = self.token_budget, []
+        for request_id in self.active:
+            if left == 0:
+                break
+            request = self.requests[request_id]
+            at = self.cache.computed[request_id]
+            most = self.prefill_chunk if at < len(request.prompt) else 1
+            count = min(most, left, request.known - at)
+            if count < 1:
+                raise RuntimeError(f'active request {request_id!r} has nothing to compute')
+            pieces.append(Work(request_id, at, request.span(at, at + count), at + count == request.known))
+            left -= count
+        served = len(pieces)
+        self.active = self.active[served:] + self.active[:served]
+        return pieces
+
+    def plan(self):
+        self._admit()
+        pieces = self._share()
+        if not pieces and self.waiting:
+            raise RuntimeError('requests are waiting, none is active and none can be admitted')
+        return pieces
