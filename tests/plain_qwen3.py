@@ -68,7 +68,7 @@ def expand_kv(t, group):
     return t[:, :, None, :].expand(T, nkv, group, d).reshape(T, nkv * group, d)
 
 
-def attention(q, k, v, positions, scale, window=None):
+def attention(q, k, v, positions, scale, window=None, key_positions=None):
     """Masked softmax attention with explicit scores.
 
     q[T, nq, d] at absolute `positions[T]`; k, v[E, nkv, d] hold positions 0..E-1.
@@ -76,7 +76,8 @@ def attention(q, k, v, positions, scale, window=None):
     iff j <= position[t] (absolute positions, qil/model.py:62-64); softmax over j;
     out[t, h] = sum_j P[h, t, j] v[j, h // g].  qil/model.py:59-68; scale :67.
     `window` (not part of Qwen3 dense; for tests of the windowed kernel) hides
-    keys with j <= position[t] - window.
+    keys with j <= position[t] - window.  `key_positions[E]` (default 0..E-1) are
+    the keys' absolute positions when the sequence does not begin at 0.
     """
     T, nq, d = q.shape
     E, nkv, _ = k.shape
@@ -86,7 +87,7 @@ def attention(q, k, v, positions, scale, window=None):
     qh = q.permute(1, 0, 2)                              # [nq, T, d]
     acc = torch.float64 if q.dtype == torch.float64 else torch.float32
     scores = (qh.to(acc) @ kh.to(acc).transpose(1, 2)) * scale
-    columns = torch.arange(E)[None, :]
+    columns = (torch.arange(E) if key_positions is None else key_positions)[None, :]
     visible = columns <= positions[:, None]
     if window is not None:
         visible = visible & (columns > positions[:, None] - window)
@@ -111,7 +112,7 @@ def attention_block(x, weights, prefix, config, positions):
     k = rms_norm(k, weights[a + 'k_norm.weight'], eps)                         # :53
     angles = rotary_angles(positions, d, theta)
     q, k = rotate(q, angles), rotate(k, angles)                                # :55
-    attended = attention(q, k, v, positions, d ** -0.5).reshape(T, nq * d)     # :65-68
+    attended = attention(q, k, v, positions, d ** -0.5, key_positions=positions).reshape(T, nq * d)     # :65-68
     return x + linear(attended, weights[a + 'o_proj.weight'], weights.get(a + 'o_proj.bias'))
 
 
@@ -183,7 +184,8 @@ def cast_weights(weights, dtype):
 
 
 def hidden_states(tokens, weights, config, start=0):
-    """Final hidden states (before the last norm) of one whole sequence.  qil/model.py:123-129."""
+    """Final hidden states (before the last norm) of one whole sequence whose first token stands at
+    position `start`.  qil/model.py:123-129."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(start, start + len(tokens))
     x = weights['model.embed_tokens.weight'][tokens]                           # :126, no scaling
@@ -198,6 +200,14 @@ def logits(tokens, weights, config, dtype=torch.float32):
     x = hidden_states(tokens, w, config)
     n = rms_norm(x, w['model.norm.weight'], config.get('rms_norm_eps', 1e-6))
     return linear(n, head_weight(w, config)).to(torch.float32)                 # :134
+
+
+def logits_at(tokens, weights, config, rows):
+    """float32 logits [len(rows), V] at the given positions only (the head is the costly part at a real
+    vocabulary); the same arithmetic as `logits`.  qil/model.py:130-134 (rows are chosen before the last norm)."""
+    x = hidden_states(tokens, weights, config)[torch.as_tensor(rows, dtype=torch.long)]
+    n = rms_norm(x, weights['model.norm.weight'], config.get('rms_norm_eps', 1e-6))
+    return linear(n, head_weight(weights, config)).to(torch.float32)
 
 
 def greedy(prompt, count, weights, config, dtype=torch.float32):

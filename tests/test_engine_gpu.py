@@ -1,6 +1,7 @@
 """Generation through the entry points, trace replay through bin/trace_run, and a toy architecture,
 on the GPU, against the plain implementation."""
 import json
+import os
 import random
 import subprocess
 import sys
@@ -119,10 +120,13 @@ def test_command_line(model_folder, tmp_path):
     assert result['token_ids'] == plain.greedy(prompt, 6, weights, config) and result['state'] == 'completed'
     assert json.loads(run.stdout[run.stdout.index('{'):])['token_ids'] == result['token_ids']
     random_folder = tmp_path / 'random'
+    elsewhere = tmp_path / 'elsewhere'                    # not the checkout's root: the package is found by its path
+    elsewhere.mkdir()
     run = subprocess.run([sys.executable, '-m', 'qil_amd', '--model', str(random_folder), '--random-config',
                           json.dumps(plain.TINY_B), '--random-seed', '3', '--token-ids', '[1, 2, 3]', '--dtype', 'bfloat16',
                           '--max-new-tokens', '4', '--temperature', '0.7', '--seed', '5', '--ignore-eos'],
-                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+                         cwd=elsewhere, env=dict(os.environ, PYTHONPATH=str(ROOT)), capture_output=True, text=True,
+                         timeout=300)
     assert run.returncode == 0, run.stderr[-2000:]
     assert len(json.loads(run.stdout[run.stdout.index('{'):])['token_ids']) == 4
     assert (random_folder / 'model.safetensors').exists()
@@ -585,6 +589,11 @@ REAL = {
                 intermediate_size=17408, num_hidden_layers=1, num_attention_heads=40, num_key_value_heads=8,
                 head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
                 attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=None),
+    # 64 query heads on a width of 5,120, an inner width of 25,600 (200 stages of 128 columns)
+    '32B': dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=151936, hidden_size=5120,
+                intermediate_size=25600, num_hidden_layers=1, num_attention_heads=64, num_key_value_heads=8,
+                head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                attention_bias=False, tie_word_embeddings=False, hidden_act='silu', eos_token_id=None),
 }
 
 
@@ -664,9 +673,10 @@ def test_portions_of_a_long_prompt_replay_a_graph_at_real_sizes(tmp_path, name, 
 
 
 @pytest.mark.parametrize('name,dtype', [('0.6B', torch.float32), ('0.6B', torch.bfloat16), ('8B', torch.bfloat16),
-                                        ('4B', torch.bfloat16), ('14B', torch.bfloat16)])
+                                        ('4B', torch.bfloat16), ('14B', torch.bfloat16), ('32B', torch.bfloat16),
+                                        ('8B', torch.float32)])
 def test_layers_of_real_size(tmp_path, name, dtype):
-    """Few layers at the sizes of Qwen3-0.6B / 4B / 8B / 14B (head size 128, vocabulary 151,936): a mixed, chunked
+    """Few layers at the sizes of Qwen3-0.6B / 4B / 8B / 14B / 32B (head size 128, vocabulary 151,936): a mixed, chunked
     replay of three requests against the plain implementation, and a greedy step through the sampler."""
     from qil_amd.engine import ModelRunner, StepEntry
     from qil_amd.sampling import Sampler, SamplingParams

@@ -591,6 +591,7 @@ def test_sampling(ops):
     vocab = 151936
     logits = rand(5, vocab, scale=2.0)
     logits[0, 70000] = logits[0, 123] = 50.0             # tie: lowest index wins (qil/engine.py:100)
+    logits[3] = logits[2]                                # the same logits, seed and temperature: only the counter differs
     temperatures = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.7]).cuda()
     seeds = torch.tensor([0, 0, 11, 11, -5], dtype=torch.int32).cuda()
     counters = torch.tensor([0, 0, 3, 4, 9], dtype=torch.int32).cuda()
@@ -600,7 +601,8 @@ def test_sampling(ops):
     scores = refs.sample_scores(logits.cpu(), temperatures.cpu(), seeds.cpu(), counters.cpu())
     for row in range(2, 5):                               # the drawn token is the reference's, or within float noise of it
         assert scores[row, tokens[row].item()] >= scores[row].max() - 1e-4
-    assert tokens[2].item() != tokens[3].item() or True  # different counters draw independently
+    assert tokens[2].item() != tokens[3].item()          # different counters draw independently (the two best scores of each row lie 0.5 apart)
+    assert scores[2].argmax().item() != scores[3].argmax().item()
     again, _ = ops.sample(logits, temperatures, seeds, counters)
     assert again.tolist() == tokens.tolist()
     logits[3, 5] = float('nan')

@@ -1,0 +1,243 @@
+"""Schedules and sizes that the benchmark configurations name, held against the plain implementation:
+decoding across the context buckets of the captured graphs, the mixed workload of 0.6B sizes in float32
+through the serving loop, and layers of 32B sizes and of 8B sizes in float32."""
+import random
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = {torch.float32: dict(atol=5e-6, rtol=5e-5), torch.bfloat16: dict(atol=0.015, rtol=0.015)}
+
+
+def random_tokens(config, length, seed):
+    r = random.Random(seed)
+    return [r.randrange(config['vocab_size']) for _ in range(length)]
+
+
+def poison(runner):
+    for group in runner.cache.kv_groups:
+        group['k'].fill_(float('nan')), group['v'].fill_(float('nan'))
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_decoding_crosses_the_graphs_context_buckets(model_folder, dtype):
+    """Three requests decode together, given tokens, the longest from 500 to 1,040 tokens: the decode graph's
+    bucket (512 tokens) changes twice, a new graph with a wider block table takes over, a request ends and
+    another takes its row.  Every logit against the plain model, and against a runner without graphs."""
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.engine import graphs as graph_module
+    from qil_amd.weights import load_model
+    config = dict(plain.TINY_B, max_position_embeddings=2560)
+    folder, weights = model_folder(config, 4)
+    model = load_model(folder, dtype=dtype, device='cuda')
+    sequences = {'a': random_tokens(config, 1040, 1), 'b': random_tokens(config, 330, 2),
+                 'c': random_tokens(config, 700, 3)}
+    heads = {'a': 500, 'b': 200, 'c': 290}
+    expected = {r: plain.logits(t, weights, config) for r, t in sequences.items()}
+    assert graph_module.BUCKET == 512
+    outputs = []
+    for with_graphs in (True, False):
+        runner = ModelRunner(model, num_pages=3 * 70, page_size=16, max_requests=3, graphs=with_graphs)
+        poison(runner)
+        fed, rows, live = {}, [], []
+
+        def begin(r):
+            runner.admit(r)
+            runner.step([StepEntry(r, tuple(sequences[r][:heads[r]]), ())])
+            fed[r] = heads[r]
+            live.append(r)
+        begin('a'), begin('b')
+        buckets, steps = set(), 0
+        while live:
+            steps += 1
+            order = live if len(rows) % 2 else live[::-1]
+            entries = [StepEntry(r, (sequences[r][fed[r]],), (0,)) for r in order]
+            buckets.add(-(-(max(fed[r] for r in order) + 1) // 512))
+            logits = runner.step(entries).cpu()
+            for i, r in enumerate(order):
+                rows.append((r, fed[r], logits[i]))
+                fed[r] += 1
+                if fed[r] == len(sequences[r]):
+                    runner.release(r)
+                    live.remove(r)
+                    if r == 'b':
+                        begin('c')                         # takes b's row of the batch and some of its pages
+        assert buckets == {1, 2, 3}
+        if with_graphs:
+            assert runner.graphs.captures >= 3 and runner.graphs.replays == steps
+        runner.cache.check()
+        assert runner.cache.free_pages == [3 * 70]
+        outputs.append(rows)
+    assert len(outputs[0]) == len(outputs[1]) > 1200
+    worst = 0.0
+    for (r, place, replayed), (r2, place2, launched) in zip(*outputs):
+        assert (r, place) == (r2, place2) and torch.isfinite(replayed).all()
+        torch.testing.assert_close(replayed, launched, **TOLERANCE[dtype], msg=lambda m: f'{r} at {place} against launches: {m}')
+        torch.testing.assert_close(replayed, expected[r][place], **TOLERANCE[dtype], msg=lambda m: f'{r} at {place}: {m}')
+        worst = max(worst, (replayed - expected[r][place]).abs().max().item())
+    print(f'{dtype}: {len(outputs[0])} rows, max abs error {worst:.2e}')
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_a_mixed_step_crosses_its_graphs_context_bucket(model_folder, dtype):
+    """Portions of 8 tokens of a long prompt beside two decoded rows while the prompt grows from 2,022 to 2,078
+    tokens: the shape's graph for contexts up to 2,048 is captured and replayed, then the next bucket's."""
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.engine import graphs as graph_module
+    from qil_amd.weights import load_model
+    config = dict(plain.TINY_B, max_position_embeddings=2560)
+    folder, weights = model_folder(config, 5)
+    model = load_model(folder, dtype=dtype, device='cuda')
+    sequences = {'p': random_tokens(config, 2078, 1), 'q': random_tokens(config, 140, 2), 'r': random_tokens(config, 67, 3)}
+    heads = {'p': 2022, 'q': 133, 'r': 60}
+    expected = {r: plain.logits(t, weights, config) for r, t in sequences.items()}
+    assert graph_module.MIXED_BUCKET == 2048
+    outputs = []
+    for with_graphs in (True, False):
+        runner = ModelRunner(model, num_pages=160, page_size=16, max_requests=3, graphs=with_graphs)
+        poison(runner)
+        fed, rows = {}, []
+        for r in 'pqr':
+            runner.admit(r)
+            runner.step([StepEntry(r, tuple(sequences[r][:heads[r]]), ())])
+            fed[r] = heads[r]
+        for turn in range(7):
+            sizes = {'p': 8, 'q': 1, 'r': 1}
+            entries = [StepEntry(r, tuple(sequences[r][fed[r]:fed[r] + sizes[r]]), (0, 7) if r == 'p' else (0,))
+                       for r in ('qpr' if turn % 2 else 'prq')]
+            logits = runner.step(entries).cpu()
+            at = 0
+            for entry in entries:
+                for w in entry.want:
+                    rows.append((entry.request, fed[entry.request] + w, logits[at]))
+                    at += 1
+                fed[entry.request] += len(entry.tokens)
+            torch.cuda.synchronize()
+        if with_graphs:
+            # per bucket: launched the first time, captured the second, replayed from then on
+            assert runner.graphs.mixed_captures == 2 and runner.graphs.mixed_replays == 5
+        outputs.append(rows)
+    assert fed == {r: len(t) for r, t in sequences.items()}
+    for (r, place, replayed), (_, _, launched) in zip(*outputs):
+        assert torch.isfinite(replayed).all()
+        torch.testing.assert_close(replayed, launched, **TOLERANCE[dtype], msg=lambda m: f'{r} at {place} against launches: {m}')
+        torch.testing.assert_close(replayed, expected[r][place], **TOLERANCE[dtype], msg=lambda m: f'{r} at {place}: {m}')
+
+
+class RecordingRunner:
+    """A ModelRunner that keeps the logits of every step (the serving loop then draws through its sampler
+    instead of inside the step)."""
+
+    def __init__(self, runner):
+        self.runner, self.cache, self.steps = runner, runner.cache, []
+
+    def step(self, entries):
+        starts = [self.cache.computed[e.request] for e in entries]
+        logits = self.runner.step(entries)
+        self.steps.append(([(e.request, s, len(e.tokens), e.want) for e, s in zip(entries, starts)],
+                           None if logits is None else logits.cpu()))
+        return logits
+
+
+MIXED_06B = dict(architectures=['Qwen3ForCausalLM'], model_type='qwen3', vocab_size=151936, hidden_size=1024,
+                 intermediate_size=3072, num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8,
+                 head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                 attention_bias=False, tie_word_embeddings=True, hidden_act='silu', eos_token_id=None)
+
+
+def test_mixed_workload_of_0p6b_sizes_in_float32(tmp_path):
+    """Eight requests of 16 to 2,048 prompt tokens through the serving loop at Qwen3-0.6B layer sizes in true
+    float32: portions of 128 under a budget of 512 tokens, 4 active at a time, 32 new tokens each, 16-token pages
+    (the protocol of benchmarks/validate_batched.py:99-173 of the reference, which holds teacher-forced logits
+    to atol = rtol = 2e-4).  Every logit the loop drew from is held against the plain model run on the request's
+    own tokens; the tokens are the plain greedy choice; the fused path of the loop produces the same tokens; all
+    pages come back."""
+    from qil_amd import Engine
+    from qil_amd.engine import ModelRunner
+    from qil_amd.weights import load_model
+    from conftest import write_model_folder
+    config = MIXED_06B
+    weights = plain.random_weights(config, 31)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.float32)
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+    r = random.Random(12)
+    lengths = [16, 2048] + [r.randint(16, 2048) for _ in range(6)]
+    r.shuffle(lengths)
+    prompts = [random_tokens(config, n, 40 + i) for i, n in enumerate(lengths)]
+    pages, new = 640, 32
+    recorder = RecordingRunner(ModelRunner(model, num_pages=pages, page_size=16, max_requests=4, max_step_tokens=512))
+    poison(recorder.runner)
+    engine = Engine(model, runner=recorder, token_budget=512, prefill_chunk=128, max_active=4)
+    results = engine.generate(prompts, max_new_tokens=new, ignore_eos=True)
+    assert all(row['state'] == 'completed' and len(row['token_ids']) == new for row in results)
+    engine.cache.check()
+    assert engine.cache.free_pages == [pages] and engine.idle
+    assert all(sum(n for _, _, n, _ in entries) <= 512 and len(entries) <= 4 for entries, _ in recorder.steps)
+    assert any(len({n for _, _, n, _ in entries}) > 1 for entries, _ in recorder.steps), 'portions beside decoded tokens'
+    drawn = {i: [] for i in range(len(prompts))}
+    for entries, logits in recorder.steps:
+        at = 0
+        for request, start, count, want in entries:
+            for w in want:
+                drawn[request].append((start + w, logits[at]))
+                at += 1
+    worst = 0.0
+    for i, (prompt, row) in enumerate(zip(prompts, results)):
+        places = [p for p, _ in drawn[i]]
+        assert places == list(range(len(prompt) - 1, len(prompt) + new - 1))
+        expected = plain.logits_at(prompt + row['token_ids'], weights, config, places)
+        got = torch.stack([l for _, l in drawn[i]])
+        assert torch.isfinite(got).all()
+        worst = max(worst, (got - expected).abs().max().item())
+        torch.testing.assert_close(got, expected, atol=2e-4, rtol=2e-4, msg=lambda m: f'request {i} ({len(prompt)} tokens): {m}')
+        for k, token in enumerate(row['token_ids']):
+            assert expected[k][token] >= expected[k].max() - 1e-4
+    print(f'0.6B sizes float32, prompts {lengths}: max abs error {worst:.2e}')
+    # the loop as it serves (the draw inside the step, graphs of decode steps): the same tokens
+    served = Engine(model, num_pages=pages, page_size=16, token_budget=512, prefill_chunk=128, max_active=4)
+    again = served.generate(prompts, max_new_tokens=new, ignore_eos=True)
+    assert [row['token_ids'] for row in again] == [row['token_ids'] for row in results]
+    stats = served.stats()
+    assert stats['drawn'] == 8 * new and stats['pages_in_use'] == [0] and stats['graph_replays'] > 0
+    assert stats['tokens'] == sum(lengths) + 8 * (new - 1) and stats['peak_pages_in_use'] <= pages
+
+
+def test_a_long_context_in_bfloat16_at_0p6b_sizes(tmp_path):
+    """A 4,000-token prompt in portions of 512 beside two decoding requests, then 24 decoded tokens at contexts
+    beyond 4,000 (bfloat16, two layers of 0.6B sizes): the logits of the last portion's end and of every decoded
+    token against the plain model."""
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.weights import load_model
+    from conftest import write_model_folder
+    config = MIXED_06B
+    weights = plain.random_weights(config, 32)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    model = load_model(folder, dtype=torch.bfloat16, device='cuda')
+    sequences = {'long': random_tokens(config, 4024, 1), 'x': random_tokens(config, 300, 2), 'y': random_tokens(config, 90, 3)}
+    runner = ModelRunner(model, num_pages=290, page_size=16, max_requests=3)
+    poison(runner)
+    fed, rows = {'long': 0, 'x': 250, 'y': 40}, {r: [] for r in sequences}
+    for r in sequences:
+        runner.admit(r)
+    for r in 'xy':
+        runner.step([StepEntry(r, tuple(sequences[r][:fed[r]]), ())])
+    while fed['long'] < len(sequences['long']):
+        size = 512 if fed['long'] < 4000 - 416 else (416 if fed['long'] < 4000 else 1)
+        entries = [StepEntry('long', tuple(sequences['long'][fed['long']:fed['long'] + size]), (size - 1,))]
+        entries += [StepEntry(r, (sequences[r][fed[r]],), (0,)) for r in 'xy' if fed[r] < len(sequences[r])]
+        logits = runner.step(entries).cpu()
+        for i, entry in enumerate(entries):
+            fed[entry.request] += len(entry.tokens)
+            rows[entry.request].append((fed[entry.request] - 1, logits[i]))
+    for r, items in rows.items():
+        places = [p for p, _ in items]
+        expected = plain.logits_at(sequences[r], weights, config, places)
+        got = torch.stack([l for _, l in items])
+        scale = max(1.0, expected.abs().max().item())
+        assert torch.isfinite(got).all()
+        print(f'{r}: {len(places)} places up to {max(places)}, max abs error {(got - expected).abs().max():.2e}, largest logit {scale:.2f}')
+        torch.testing.assert_close(got, expected, atol=0.015 * scale, rtol=0.02)

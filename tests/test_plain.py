@@ -149,3 +149,147 @@ def test_sampling_reference():
     assert plain.sample(row, 0.9, 5, 11)[0] == plain.sample(row, 0.9, 5, 11)[0]
     u = plain.gumbel_uniform(1, 2, 1000)
     assert 0 < u.min() and u.max() < 1 and abs(u.mean() - 0.5) < 0.05
+
+
+# ---------------------------------------------------------------- where the norms sit, which branch is gated, the output bias
+# The reference pins these against a library model (tests/qil/test_model.py:19-33); that model's code is not a
+# source here, so each reading of qil/model.py:35,52-55,71 is pinned by an invariant that only it satisfies, and
+# every test below first shows that the plausible other reading breaks the invariant.
+
+def _attention_variant(x, weights, prefix, config, positions, norm_after_rotation=False, norm_v=False):
+    """qil/model.py:48-69 from the plain parts, with the two misreadings as switches."""
+    nq, nkv, d = config['num_attention_heads'], config['num_key_value_heads'], config['head_dim']
+    eps, theta, T = config['rms_norm_eps'], config['rope_theta'], x.shape[0]
+    a = prefix + 'self_attn.'
+    n = plain.rms_norm(x, weights[prefix + 'input_layernorm.weight'], eps)
+    q = plain.linear(n, weights[a + 'q_proj.weight']).reshape(T, nq, d)
+    k = plain.linear(n, weights[a + 'k_proj.weight']).reshape(T, nkv, d)
+    v = plain.linear(n, weights[a + 'v_proj.weight']).reshape(T, nkv, d)
+    angles = plain.rotary_angles(positions, d, theta)
+    if norm_after_rotation:
+        q = plain.rms_norm(plain.rotate(q, angles), weights[a + 'q_norm.weight'], eps)
+        k = plain.rms_norm(plain.rotate(k, angles), weights[a + 'k_norm.weight'], eps)
+    else:
+        q = plain.rotate(plain.rms_norm(q, weights[a + 'q_norm.weight'], eps), angles)
+        k = plain.rotate(plain.rms_norm(k, weights[a + 'k_norm.weight'], eps), angles)
+    if norm_v:
+        v = plain.rms_norm(v, weights[a + 'k_norm.weight'], eps)
+    out = plain.attention(q, k, v, positions, d ** -0.5, key_positions=positions).reshape(T, nq * d)
+    return x + plain.linear(out, weights[a + 'o_proj.weight'])
+
+
+def _uneven_norms(config, seed):
+    """Random weights whose q/k norm weights differ a lot from one dimension to the next (a rotation of a pair
+    then no longer commutes with the weights)."""
+    weights = plain.random_weights(config, seed, std=0.2, round_to=None)
+    g = torch.Generator().manual_seed(seed + 100)
+    for name in weights:
+        if name.endswith('q_norm.weight') or name.endswith('k_norm.weight'):
+            weights[name] = 0.3 + 2.0 * torch.rand(weights[name].shape, generator=g)
+    return {k: v.double() for k, v in weights.items()}
+
+
+def test_qk_norm_comes_before_the_rotation():
+    """Scores may depend on distances only (a shift of every position changes nothing).  With the norm's
+    per-dimension weights applied after the rotation that fails; with the norm first it holds."""
+    config = dict(plain.TINY_A, rope_theta=100.0)
+    weights = _uneven_norms(config, 5)
+    tokens = torch.tensor([5, 17, 3, 200, 41, 8, 99])
+    x = weights['model.embed_tokens.weight'][tokens]
+    here, there = torch.arange(7), torch.arange(7) + 37
+    prefix = 'model.layers.0.'
+    torch.testing.assert_close(plain.attention_block(x, weights, prefix, config, here),
+                               plain.attention_block(x, weights, prefix, config, there), atol=1e-5, rtol=1e-5)   # angles are float32
+    # the variant function is the plain block when its switches are off ...
+    torch.testing.assert_close(_attention_variant(x, weights, prefix, config, here),
+                               plain.attention_block(x, weights, prefix, config, here), atol=1e-12, rtol=1e-12)
+    # ... and the other order is no function of distances
+    wrong = _attention_variant(x, weights, prefix, config, here, norm_after_rotation=True)
+    wrong_shifted = _attention_variant(x, weights, prefix, config, there, norm_after_rotation=True)
+    assert (wrong - wrong_shifted).abs().max() > 1e-2
+    # the whole model inherits the invariance
+    torch.testing.assert_close(plain.hidden_states(tokens, weights, config, start=0),
+                               plain.hidden_states(tokens, weights, config, start=211), atol=1e-4, rtol=1e-4)
+
+
+def test_queries_and_keys_are_normalised_per_head_and_values_are_not():
+    config = dict(plain.TINY_B, rms_norm_eps=1e-30)
+    weights = _uneven_norms(config, 6)
+    tokens = torch.tensor([5, 17, 3, 200, 41])
+    x = weights['model.embed_tokens.weight'][tokens]
+    prefix, positions, d = 'model.layers.1.', torch.arange(5), config['head_dim']
+    base = plain.attention_block(x, weights, prefix, config, positions) - x
+    assert base.abs().max() > 1e-3
+
+    def changed(name, rows, factor):
+        w = dict(weights)
+        t = w[prefix + name].clone()
+        t[rows] *= factor
+        w[prefix + name] = t
+        return plain.attention_block(x, w, prefix, config, positions) - x
+    # one query head and one key head scaled: nothing changes (norm over that head's d elements alone);
+    # a norm over the whole q width, or none, would change the scores
+    torch.testing.assert_close(changed('self_attn.q_proj.weight', slice(2 * d, 3 * d), 7.0), base, atol=1e-10, rtol=1e-9)
+    torch.testing.assert_close(changed('self_attn.k_proj.weight', slice(d, 2 * d), 0.2), base, atol=1e-10, rtol=1e-9)
+    # half a head scaled: the norm is over the whole head, so this does change the result
+    assert (changed('self_attn.q_proj.weight', slice(2 * d, 2 * d + d // 2), 7.0) - base).abs().max() > 1e-5
+    # values pass as they are: the sub-layer's output is linear in v_proj
+    torch.testing.assert_close(changed('self_attn.v_proj.weight', slice(None), 3.0), 3.0 * base, atol=1e-10, rtol=1e-9)
+    normalised_v = _attention_variant(x, weights, prefix, config, positions, norm_v=True) - x
+    assert (normalised_v - base).abs().max() > 1e-4
+
+
+def test_the_gate_branch_takes_the_activation():
+    """silu(gate) * up: linear in the up branch, zero where the gate is very negative, about up where the gate is
+    large and positive times itself.  The other pairing (gate * silu(up)) fails each of the three."""
+    g = torch.Generator().manual_seed(3)
+    n = torch.randn(4, 10, generator=g, dtype=torch.float64)
+    gate, up, down = (torch.randn(s, generator=g, dtype=torch.float64) for s in ((6, 10), (6, 10), (10, 6)))
+    base = plain.gated_mlp(n, gate, up, down)
+    torch.testing.assert_close(plain.gated_mlp(n, gate, -2.5 * up, down), -2.5 * base)       # odd and linear in up
+    assert not torch.allclose(plain.gated_mlp(n, -2.5 * gate, up, down), -2.5 * base)        # but not in gate
+    # a gate whose pre-activations are all -40: silu gives ~0 whatever the up branch holds
+    positive = torch.rand(4, 10, generator=g, dtype=torch.float64) + 0.5
+    closed = -40.0 / positive.sum(-1).min() * torch.ones(6, 10, dtype=torch.float64)
+    assert (positive @ closed.T).max() <= -40.0 + 1e-9
+    assert plain.gated_mlp(positive, closed, up, down).abs().max() < 1e-12
+    assert plain.gated_mlp(positive, up, closed, down).abs().max() > 1e-3                     # roles swapped: not zero
+    # a wide-open gate: silu(z) -> z, so the result is (n gate^T) * (n up^T) down^T
+    open_gate = -closed
+    z = positive @ open_gate.T
+    torch.testing.assert_close(plain.gated_mlp(positive, open_gate, up, down), (z * (positive @ up.T)) @ down.T)
+
+
+def test_attention_bias_reaches_all_four_projections():
+    """qil/model.py:32-35: ``attention_bias`` gives q, k, v and the output projection a bias each."""
+    config = plain.TINY_C
+    shapes = plain.tensor_shapes(config)
+    for name in ('q_proj', 'k_proj', 'v_proj', 'o_proj'):
+        assert f'model.layers.0.self_attn.{name}.bias' in shapes
+    assert not any(name.endswith('.bias') for name in plain.tensor_shapes(plain.TINY_A))
+    weights = plain.random_weights(config, 2)
+    g = torch.Generator().manual_seed(8)
+    for name in weights:
+        if name.endswith('.bias'):
+            weights[name] = torch.randn(weights[name].shape, generator=g)
+    tokens = torch.tensor([1, 2, 3, 4])
+    x = weights['model.embed_tokens.weight'][tokens]
+    prefix = 'model.layers.0.'
+    silent = dict(weights)
+    silent[prefix + 'self_attn.o_proj.weight'] = torch.zeros_like(weights[prefix + 'self_attn.o_proj.weight'])
+    out = plain.attention_block(x, silent, prefix, config, torch.arange(4)) - x
+    torch.testing.assert_close(out, weights[prefix + 'self_attn.o_proj.bias'].expand(4, -1))  # the output bias alone
+    # a value bias b_v alone (W_v = 0): every head attends to the constant b_v, the block gives W_o b_v + b_o
+    constant = dict(weights)
+    constant[prefix + 'self_attn.v_proj.weight'] = torch.zeros_like(weights[prefix + 'self_attn.v_proj.weight'])
+    group = config['num_attention_heads'] // config['num_key_value_heads']
+    b_v = weights[prefix + 'self_attn.v_proj.bias'].reshape(config['num_key_value_heads'], -1)
+    spread = b_v.repeat_interleave(group, 0).reshape(-1)
+    expected = weights[prefix + 'self_attn.o_proj.weight'] @ spread + weights[prefix + 'self_attn.o_proj.bias']
+    torch.testing.assert_close(plain.attention_block(x, constant, prefix, config, torch.arange(4)) - x,
+                               expected.expand(4, -1), atol=1e-5, rtol=1e-4)
+    # q and k biases change the scores: the result moves when they are dropped
+    dropped = {k: (torch.zeros_like(v) if k.endswith('q_proj.bias') or k.endswith('k_proj.bias') else v)
+               for k, v in weights.items()}
+    assert not torch.allclose(plain.attention_block(x, dropped, prefix, config, torch.arange(4)),
+                              plain.attention_block(x, weights, prefix, config, torch.arange(4)), atol=1e-4)
