@@ -154,8 +154,18 @@ class DecodeGraphs:
         return self._safe
 
     def takes(self, entries):
-        return self.safe() and all(len(e[1] if not isinstance(e, StepEntry) else e.tokens) == 1 and
-                   tuple(e[2] if not isinstance(e, StepEntry) else e.want) == (0,) for e in entries) and len(entries) > 0
+        """A decode batch: every entry brings one token and wants its logits (entries may be plain tuples, whose
+        third member, the wanted places, may be missing)."""
+        if not entries or not self.safe():
+            return False
+        for entry in entries:
+            if isinstance(entry, StepEntry):
+                tokens, want = entry.tokens, entry.want
+            else:
+                tokens, want = entry[1], (entry[2] if len(entry) > 2 else ())
+            if len(tokens) != 1 or tuple(want) != (0,):
+                return False
+        return True
 
     def mixed_step(self, entries):
         """(logits, entries, starts) of a step with prompt portions from a graph of its shape, or None: the shape

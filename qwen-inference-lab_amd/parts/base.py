@@ -103,8 +103,11 @@ class Mixer(Part):
     cache view of its schedule entry (cache/manager.py: KVView or StateView).
     Its result must not depend on how a request's tokens were cut into steps.
     """
-    # True if forward reads only device tensors of the step context (and shapes), never its host
-    # lists: then a decode step may be captured into a HIP graph and replayed with other contents.
+    # True if (1) forward reads only device tensors of the step context (and shapes), never its host
+    # lists, and (2) running forward twice on the same step leaves the cache as running it once does
+    # (writing the step's keys and values again is such; adding into a state is not): then a step may
+    # be captured into a HIP graph and replayed with other contents.  A new graph runs its first step
+    # once launch by launch and once more as the first replay.
     graph_safe = False
 
     def cache_need(self):

@@ -713,7 +713,11 @@ def test_layers_of_real_size(tmp_path, name, dtype):
         # in bfloat16 with the reference's rounding places is 0.040 away from float32 on this very model,
         # largest logit 3.4; the tiny models' 0.015 is the same bound at a largest logit of about 1.)
         scale = max(1.0, expected.abs().max().item())
-        tolerance = dict(atol=2e-5, rtol=2e-4) if dtype == torch.float32 else dict(atol=0.015 * scale, rtol=0.02)
+        # float32: only the order of the sums differs; the bound is 2e-5 at the 0.6B sizes' logits (std 0.64) and
+        # goes with the size of the logits (the reference's own float32 bound at real sizes is 2e-4,
+        # benchmarks/validate_batched.py:114)
+        tolerance = dict(atol=2e-5 * max(1.0, expected.std().item() / 0.64), rtol=2e-4) if dtype == torch.float32 \
+            else dict(atol=0.015 * scale, rtol=0.02)
         got = torch.stack([row for _, row in items]).cpu()
         want = expected[[p for p, _ in items]]
         assert torch.isfinite(got).all()

@@ -587,6 +587,103 @@ def test_one_far_key_among_hundreds(ops):
         torch.testing.assert_close(got[0, h * d:(h + 1) * d].cpu(), histories[0][1][target, kvh], atol=1e-4, rtol=1e-4)
 
 
+def pointed_queries(histories, row_seq, targets, heads, kv_heads, d, dtype):
+    """Queries whose every head points, 200 long, along the key `targets[r]` of its kv head in row r's history:
+    that key's score then stands out by hundreds, the softmax is one-hot and the output is that key's value."""
+    q = torch.zeros(len(targets), heads, d)
+    for r, (s, target) in enumerate(zip(row_seq, targets)):
+        for h in range(heads):
+            key = histories[s][0][target, h // (heads // kv_heads)].float()
+            q[r, h] = 200.0 * key / key.norm()
+    return q.reshape(len(targets), heads * d).to(dtype).cuda()
+
+
+def values_of(histories, row_seq, targets, heads, kv_heads):
+    return torch.stack([histories[s][1][t].float().repeat_interleave(heads // kv_heads, 0).reshape(-1)
+                        for s, t in zip(row_seq, targets)])
+
+
+def test_decode_kernel_finds_one_key_at_the_edges_of_its_parts(ops):
+    """bfloat16 matrix-core decode kernel, context in nine parts of 256 keys: a key at 0, at the ends of a 32-key
+    step, at the last place of a part, at the first of the next, and the newest key, each dominant for one row."""
+    page_size, d, heads, kv_heads, n = 16, 128, 8, 2, 2100
+    targets = [0, 31, 32, 255, 256, 1023, 1024, 2047, 2048, n - 1]
+    rows = len(targets)
+    k_cache, v_cache, table, histories = build_cache([n] * rows, page_size, kv_heads, d, torch.bfloat16)
+    part, parts = ops._decode_parts(rows, kv_heads, n)
+    assert part == 256 and parts == 9 and ops.library.load().qil_attn_decode_takes(heads, kv_heads, d, page_size)
+    row_seq = list(range(rows))
+    q = pointed_queries(histories, row_seq, targets, heads, kv_heads, d, torch.bfloat16)
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
+                block_tables=table, positions=torch.full((rows,), n - 1, dtype=torch.int32).cuda(),
+                row_seq=torch.arange(rows, dtype=torch.int32).cuda(), cu_seqlens=None, seq_starts=None, single_rows=None,
+                n_seqs=rows, max_query=1, max_context=n, scale=1.0, window=None)
+    want = values_of(histories, row_seq, targets, heads, kv_heads)
+    torch.testing.assert_close(ops.paged_attention(q, **args).float().cpu(), want, atol=1e-6, rtol=0)
+    lazy = ops.paged_attention(q, unmerged=True, **args)                      # merged by the output projection's kernel
+    assert isinstance(lazy, ops.Unmerged)
+    torch.testing.assert_close(lazy.merge().float().cpu(), want, atol=1e-6, rtol=0)
+
+
+def test_fused_decode_kernel_finds_one_key_also_the_one_in_registers(ops):
+    """The decode kernel that makes its own queries (no norm and no rotation here, so the queries can be aimed):
+    dominant keys at the edges of parts and steps in the pages, and the step's own new key, which the kernel
+    holds in registers and writes into the pages."""
+    page_size, d, heads, kv_heads, n = 16, 128, 8, 2, 1500
+    targets = [0, 255, 256, 511, 512, 1471, 1472, n - 2, n - 1, n - 1]
+    rows, total = len(targets), heads + 2 * kv_heads
+    k_cache, v_cache, table, histories = build_cache([n] * rows, page_size, kv_heads, d, torch.bfloat16)
+    row_seq = list(range(rows))
+    q = pointed_queries(histories, row_seq, targets, heads, kv_heads, d, torch.float32)
+    new_k = torch.stack([h[0][n - 1].float().reshape(-1) for h in histories]).cuda()        # the newest token's key and value
+    new_v = torch.stack([h[1][n - 1].float().reshape(-1) for h in histories]).cuda()
+    whole = torch.cat([q, new_k, new_v], dim=1)
+    qkv = ops.Partials(torch.stack([0.25 * whole, 0.75 * whole]).contiguous())                # two partial sums of it
+    positions = torch.full((rows,), n - 1, dtype=torch.int32).cuda()
+    j = n - 1
+    k_cache[table[:, j // page_size].long(), :, j % page_size] = float('nan')                 # the pages do not hold it yet
+    v_cache[table[:, j // page_size].long(), :, :, j % page_size] = float('nan')
+    sizes = dict(heads=heads, kv_heads=kv_heads, head_dim=d)
+    assert ops.decode_attention_takes(qkv, page_size=page_size, rotation=None, dtype=torch.bfloat16, **sizes)
+    assert ops._decode_parts(rows, kv_heads, n)[1] > 1
+    got = ops.decode_attention(qkv, q_weight=None, k_weight=None, eps=0.0, rotation=None, positions=positions, writes=True,
+                               k_cache=k_cache, v_cache=v_cache, page_size=page_size, block_tables=table,
+                               row_seq=torch.arange(rows, dtype=torch.int32).cuda(), max_context=n, scale=1.0, window=None,
+                               **sizes)
+    torch.testing.assert_close(got.float().cpu(), values_of(histories, row_seq, targets, heads, kv_heads), atol=1e-6, rtol=0)
+    written = k_cache[table[:, j // page_size].long(), :, j % page_size].float().cpu()
+    torch.testing.assert_close(written, torch.stack([h[0][j].float() for h in histories]), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize('length,chunk,split', [(700, 100, (64, 2)), (300, 300, None), (2048, 128, None)])
+def test_prompt_kernels_find_one_key_at_the_edges_of_tiles_and_parts(ops, monkeypatch, length, chunk, split):
+    """bfloat16 prompt attention (32 x 32 tiles; keys in one piece or in parts that are merged): every row aims at
+    one key, in turn the first, the ends of 32- and 64-key tiles, its own key and the one before it."""
+    page_size, d, heads, kv_heads = 16, 128, 4, 2
+    if split is not None:
+        monkeypatch.setattr(ops, 'TILE_KEY_PARTS', split)
+    k_cache, v_cache, table, histories = build_cache([length], page_size, kv_heads, d, torch.bfloat16)
+    start = length - chunk
+    fixed = [0, 31, 32, 63, 64, 127, 128, 191, 192]
+    targets = []
+    for i in range(chunk):
+        position = start + i
+        choices = [t for t in fixed + [start - 1, start] if 0 <= t <= position] + [position, max(position - 1, 0)]
+        targets.append(choices[i % len(choices)])
+    row_seq = [0] * chunk
+    q = pointed_queries(histories, row_seq, targets, heads, kv_heads, d, torch.bfloat16)
+    dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
+    if split is None and length > 1000:
+        parts = ops.tile_key_parts(ops.library.load(), torch.bfloat16, 1, chunk, heads, kv_heads, d, page_size,
+                                   table.shape[1], length)[1]
+        assert parts > 1, 'a portion deep in a context: the split is chosen by itself'
+    got = ops.paged_attention(q, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                              page_size=page_size, block_tables=table, row_seq=dev(row_seq),
+                              positions=dev(list(range(start, length))), cu_seqlens=dev([0, chunk]), seq_starts=dev([start]),
+                              single_rows=dev([]), n_seqs=1, max_query=chunk, max_context=length, scale=1.0, window=None)
+    torch.testing.assert_close(got.float().cpu(), values_of(histories, row_seq, targets, heads, kv_heads), atol=1e-6, rtol=0)
+
+
 def test_sampling(ops):
     vocab = 151936
     logits = rand(5, vocab, scale=2.0)

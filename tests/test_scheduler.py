@@ -185,3 +185,32 @@ def test_scheduler_rejects_nonsense():
     scheduler.add(Request(0, [1], 1, frozenset(), 0.0))
     with pytest.raises(ValueError, match='duplicate'):
         scheduler.add(Request(0, [1], 1, frozenset(), 0.0))
+
+
+def test_counters_of_the_loop():
+    e, runner = engine(token_budget=6, prefill_chunk=4, max_active=2)
+    assert e.stats()['steps'] == 0 and e.stats()['pages_in_use'] == [0]
+    e.submit([1] * 9, max_new_tokens=2, ignore_eos=True)
+    e.submit([2] * 3, max_new_tokens=3, ignore_eos=True)
+    e.submit([3], max_new_tokens=1, ignore_eos=True)
+    e.step()
+    stats = e.stats()
+    assert stats['steps'] == 1 and stats['last_step_tokens'] == 6 and stats['last_step_requests'] == 2
+    assert stats['active'] == 2 and stats['waiting'] == 1 and stats['drawn'] == 0
+    assert stats['pages_in_use'] == [2] and stats['pages_total'] == [16]      # 4 + 2 tokens in pages of 4
+    while not e.idle:
+        e.step()
+    stats = e.stats()
+    assert stats['tokens'] == (9 + 1) + (3 + 2) + 1 and stats['drawn'] == 6   # fed: prompts and all drawn tokens but the last
+    assert stats['pages_in_use'] == [0] and stats['peak_pages_in_use'] >= 4 and stats['active'] == stats['waiting'] == 0
+
+
+def test_requests_report_phases():
+    from qil_amd.engine import Phase
+    e, _ = engine()
+    rid = e.submit([1, 2], max_new_tokens=1, ignore_eos=True)
+    request = e.scheduler.requests[rid]
+    assert request.phase is Phase.WAITING and e.result(rid)['state'] == 'waiting' and e.result(rid)['ttft_s'] is None
+    e.step()
+    assert request.phase is Phase.COMPLETED and e.result(rid)['finish_reason'] == 'length'
+    assert request.span(0, 3) == (1, 2, follow(2, 1)[0]) and request.span(2, 3) == (follow(2, 1)[0],)

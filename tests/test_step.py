@@ -205,6 +205,17 @@ def test_long_decoding_crosses_attention_splits(case):
     case.close(torch.cat(got), plain.logits(tokens, weights, config)[199:])
 
 
+def test_which_steps_a_decode_graph_takes(model_folder, cpu_kernels):
+    from qil_amd.engine.graphs import DecodeGraphs
+    folder, _ = model_folder(plain.TINY_A, 0)
+    runner = ModelRunner(load_model(folder, dtype=torch.float32, device='cpu'), num_pages=4, page_size=4)
+    graphs = DecodeGraphs(runner)
+    assert graphs.takes([StepEntry('a', (1,), (0,)), ('b', [2], [0])])
+    assert not graphs.takes([('a', [1])])                       # nothing wanted (the third member may be missing)
+    assert not graphs.takes([StepEntry('a', (1, 2), (1,))]) and not graphs.takes([StepEntry('a', (1,), ())])
+    assert not graphs.takes([])
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 def test_graph_replays_equal_eager_launches(model_folder, dtype):
