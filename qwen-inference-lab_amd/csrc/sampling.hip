@@ -7,6 +7,8 @@
 // uniform in (0, 1) keyed by (seed, output index, i), so a request's draws depend neither on the
 // batch it sits in nor on how its work was cut.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16; x *= 0x7feb352du;
@@ -101,12 +103,11 @@ size_t qil_sample_workspace(int rows, int vocab) {
   return (size_t)rows * ((vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK) * 12;
 }
 
-int qil_sample(const float* logits, const float* temperatures, const int* seeds, const int* counters, int* tokens,
-               int* finite, void* workspace, int rows, int vocab, hipStream_t s) {
-  if (rows == 0) return 0;
-  if (rows > 65535) return -1;
+// The two launches of a draw over scratch memory that holds, per (row, chunk) cell, a value, an index and a flag.
+static int launch_sample(const float* logits, const float* temperatures, const int* seeds, const int* counters,
+                         int* tokens, int* finite, void* scratch_memory, int rows, int vocab, hipStream_t s) {
   const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
-  float* values = (float*)workspace;
+  float* values = (float*)scratch_memory;
   int* indices = (int*)(values + (size_t)rows * chunks);
   int* bad = indices + (size_t)rows * chunks;
   hipLaunchKernelGGL(sample_scan_kernel, dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, s, logits, temperatures, seeds,
@@ -114,6 +115,61 @@ int qil_sample(const float* logits, const float* temperatures, const int* seeds,
   hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, s, values, indices, bad, tokens, finite,
                      chunks);
   QIL_RETURN_LAUNCH_STATUS();
+}
+
+int qil_sample(const float* logits, const float* temperatures, const int* seeds, const int* counters, int* tokens,
+               int* finite, void* workspace, int rows, int vocab, hipStream_t s) {
+  if (rows == 0) return 0;
+  if (rows > 65535) return -1;
+  return launch_sample(logits, temperatures, seeds, counters, tokens, finite, workspace, rows, vocab, s);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------- the variant that allocates nothing
+// Scratch memory of qil_sample_static.  In host code this name is only a handle for hipGetSymbolAddress, never a
+// device address: the kernels get the looked-up address of the current device's copy.
+static __device__ __align__(256) unsigned char scratch[(size_t)QIL_SAMPLE_STATIC_CELLS * 12];
+
+#define QIL_MAX_DEVICES 64
+static void* scratch_address[QIL_MAX_DEVICES];     // per device: where its copy of `scratch` lies (null: not looked up)
+static std::mutex scratch_lock;
+
+// The current device's copy of `scratch` (looked up once per device, with that device current); 0 or a HIP error.
+static int scratch_of_current_device(void** address) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return (int)status;
+  if (device < 0 || device >= QIL_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_address[device] == nullptr) {
+    void* found = nullptr;
+    status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (status != hipSuccess) return (int)status;
+    if (found == nullptr) return (int)hipErrorInvalidSymbol;
+    scratch_address[device] = found;
+  }
+  *address = scratch_address[device];
+  return 0;
+}
+
+extern "C" {
+
+int qil_sample_static_prepare(void) {
+  void* address = nullptr;
+  return scratch_of_current_device(&address);
+}
+
+int qil_sample_static(const float* logits, const float* temperatures, const int* seeds, const int* counters,
+                      int* tokens, int* finite, int rows, int vocab, hipStream_t s) {
+  if (rows == 0) return 0;
+  if (rows < 0 || vocab < 1 || rows > 65535) return -1;
+  const long long chunks = ((long long)vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  if ((long long)rows * chunks > QIL_SAMPLE_STATIC_CELLS) return -2;
+  void* address = nullptr;
+  const int status = scratch_of_current_device(&address);
+  if (status) return status;
+  return launch_sample(logits, temperatures, seeds, counters, tokens, finite, address, rows, vocab, s);
 }
 
 }  // extern "C"

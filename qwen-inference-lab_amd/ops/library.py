@@ -178,6 +178,10 @@ def _declare(lib):
     lib.qil_sample.argtypes = [p, p, p, p, p, p, p, i, i, p]
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z
+    lib.qil_sample_static.argtypes = [p, p, p, p, p, p, i, i, p]
+    lib.qil_sample_static.restype = i
+    lib.qil_sample_static_prepare.argtypes = []
+    lib.qil_sample_static_prepare.restype = i
     for name in ('qil_embed', 'qil_add_rmsnorm', 'qil_silu_mul', 'qil_add_bias', 'qil_qk_norm_rope_store',
                  'qil_attn_rows', 'qil_attn_merge', 'qil_attn_decode', 'qil_attn_decode_fused', 'qil_attn_tile', 'qil_gemm_f32', 'qil_gemm_bf16', 'qil_gemm_bf16_gated', 'qil_gemm_bf16_unmerged', 'qil_sample'):
         getattr(lib, name).restype = i

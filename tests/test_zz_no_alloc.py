@@ -1,0 +1,67 @@
+"""The draw that allocates nothing (``qil_sample_static``: scratch memory inside the library's device image),
+called through ctypes, against ``qil_sample`` with a workspace of the caller's."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_static_draw_matches_the_draw_with_a_workspace():
+    from qil_amd.ops import library
+    lib = library.load()
+    p, i = ctypes.c_void_p, ctypes.c_int
+    lib.qil_sample_static.argtypes = [p, p, p, p, p, p, i, i, p]
+    lib.qil_sample_static.restype = i
+    lib.qil_sample_static_prepare.argtypes = []
+    lib.qil_sample_static_prepare.restype = i
+    device = torch.device('cuda:0')
+    stream = torch.cuda.current_stream(device).cuda_stream
+    assert lib.qil_sample_static_prepare() == 0
+    generator = torch.Generator().manual_seed(5)
+
+    def case(rows, vocab):
+        logits = (torch.randn(rows, vocab, generator=generator) * 2).to(device)
+        logits[0, vocab // 3] = logits[0, 5] = 60.0                         # a tie: the lowest index
+        temperatures = torch.tensor([0.0 if r % 2 == 0 else 0.5 + 0.1 * r for r in range(rows)], device=device)
+        seeds = torch.arange(rows, dtype=torch.int32, device=device) * 7 - 3
+        counters = torch.arange(rows, dtype=torch.int32, device=device) + 2
+        if rows > 2:
+            logits[2, vocab - 1] = float('nan')                             # flagged, not drawn from
+        return logits, temperatures, seeds, counters
+
+    def with_workspace(logits, temperatures, seeds, counters):
+        rows, vocab = logits.shape
+        out = torch.full((2, rows), -7, dtype=torch.int32, device=device)
+        workspace = torch.empty(lib.qil_sample_workspace(rows, vocab) // 4, dtype=torch.int32, device=device)
+        assert lib.qil_sample(logits.data_ptr(), temperatures.data_ptr(), seeds.data_ptr(), counters.data_ptr(),
+                              out[0].data_ptr(), out[1].data_ptr(), workspace.data_ptr(), rows, vocab, stream) == 0
+        return out
+
+    def static(logits, temperatures, seeds, counters):
+        rows, vocab = logits.shape
+        out = torch.full((2, rows), -7, dtype=torch.int32, device=device)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated(device)
+        status = lib.qil_sample_static(logits.data_ptr(), temperatures.data_ptr(), seeds.data_ptr(), counters.data_ptr(),
+                                       out[0].data_ptr(), out[1].data_ptr(), rows, vocab, stream)
+        assert status == 0 and torch.cuda.memory_allocated(device) == before
+        return out
+
+    # two calls in a row on the same scratch memory, the second smaller (fewer rows and fewer chunks a row):
+    # what the first left behind must not show
+    for rows, vocab in ((9, 151936), (4, 5000), (1, 37)):
+        inputs = case(rows, vocab)
+        expected, got = with_workspace(*inputs), static(*inputs)
+        torch.cuda.synchronize()
+        assert got.tolist() == expected.tolist(), (rows, vocab)
+        assert expected[0, 0].item() == 5 and (rows < 3 or expected[1].tolist()[2] == 0)
+    # sizes beyond the scratch memory are refused, not run: 65,536 cells of 4,096 logits
+    inputs = case(2, 64)
+    out = torch.zeros((2, 2), dtype=torch.int32, device=device)
+    args = [t.data_ptr() for t in inputs] + [out[0].data_ptr(), out[1].data_ptr()]
+    assert lib.qil_sample_static(*args, 1725, 151936, stream) == -2          # 1,725 * 38 chunks > 65,536
+    assert lib.qil_sample_static(*args, 70000, 64, stream) == -1
+    assert lib.qil_sample_static(*args, 0, 64, stream) == 0
+    torch.cuda.synchronize()
