@@ -229,10 +229,24 @@ __device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
                     pack_bf16(numer[4] / denom, numer[5] / denom), pack_bf16(numer[6] / denom, numer[7] / denom));
 }
 
-template <typename OUT, bool MERGE>
+// A given as the float32 residual stream whose RMSNorm is to be taken (qil/model.py:15-23), with the rows' sums of
+// squares already there in pieces: squares [pieces][M], one piece per 16 columns of the stream, left by the kernel that
+// completed the stream (gemm_bf16_cols.hip).  The block adds the pieces in a fixed order, normalises its slice of the
+// row (round, then the weight, as add_rmsnorm in elementwise.hip does) and needs no norm kernel before it.
+struct NormedA {
+  const float* stream;                                     // [M, K]
+  const float* weight;                                     // [K]
+  const float* squares;                                    // [pieces][M]
+  int pieces;
+  float eps;
+};
+
+// ASRC: 0 = A as it is, 1 = merged attention parts (UnmergedA), 2 = normalised stream (NormedA)
+template <typename OUT, int ASRC>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
-gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const bf16_t* __restrict__ W,
+gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, NormedA normed, const bf16_t* __restrict__ W,
                        OUT* __restrict__ C, int M, int N, int K, int cols_per_split) {
+  constexpr bool MERGE = ASRC == 1;
   extern __shared__ __align__(16) bf16_t lds[];            // A slice [8 or 16][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
@@ -253,11 +267,37 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
     place[u] = row * 128 + ((piece ^ row) & 15) * 8;
   }
   // A slice first: its wait would otherwise cover the first stages of W as well
-  for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
-    const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (m < M) v = MERGE ? merged8(unmerged, m, k_begin + c) : *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
-    *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+  if (ASRC == 2) {
+    // 1 / rms of the rows: wave m (and m + 8) adds the row's pieces lane by lane, then across the wave
+    float* rstd = reinterpret_cast<float*>(lds + a_rows * row_width + LINES_WAVES * (16 * 128));
+    for (int m = wave; m < M; m += LINES_WAVES) {
+      float sum = 0.f;
+      for (int p = lane; p < normed.pieces; p += QIL_WAVE) sum += normed.squares[(size_t)p * M + m];
+      sum = wave_sum(sum);
+      if (lane == 0) rstd[m] = rsqrtf(sum / (float)K + normed.eps);
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
+      const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (m < M) {
+        float x[8], g[8];
+        ld8(normed.stream + (size_t)m * K + k_begin + c, x);
+        ld8(normed.weight + k_begin + c, g);
+        const float scale = rstd[m];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = round_to<bf16_t>(x[e] * scale) * g[e];
+        v = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+      }
+      *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
+      const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (m < M) v = MERGE ? merged8(unmerged, m, k_begin + c) : *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
+      *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+    }
   }
   // Every wave walks its K range from a start of its own and wraps around: waves that all read the
   // same columns of their rows at the same time load a few memory channels only.
@@ -317,7 +357,7 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, const b
 
 static size_t lines_lds(int M, int K, int splits) {
   const int rows = M <= 8 ? 8 : 16;
-  return ((size_t)rows * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
+  return ((size_t)rows * (K / splits + GEMM_LDS_PAD) + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t) + 16 * sizeof(float);
 }
 
 // Whether the whole-line kernel takes the product with this many splits.
@@ -328,11 +368,11 @@ static bool lines_takes(const void* A, const void* W, const float* bias, int M, 
   return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
 }
 
-template <typename OUT, bool MERGE = false>
+template <typename OUT, int ASRC = 0>
 static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s,
-                        UnmergedA unmerged = UnmergedA()) {
+                        UnmergedA unmerged = UnmergedA(), NormedA normed = NormedA()) {
   const size_t lds = lines_lds(M, K, splits);
-  auto kernel = gemm_bf16_lines_kernel<OUT, MERGE>;
+  auto kernel = gemm_bf16_lines_kernel<OUT, ASRC>;
   static size_t granted = 0;                              // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -340,7 +380,7 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
     granted = lds;
   }
   dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
-  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, unmerged, W, C, M, N, K, K / splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, unmerged, normed, W, C, M, N, K, K / splits);
   return 0;
 }
 
@@ -819,7 +859,28 @@ extern "C" int qil_gemm_bf16_unmerged(const void* workspace, const int* position
   u.l = u.m + (size_t)M * heads * parts;
   u.positions = positions;
   u.heads = heads; u.d = d; u.parts = parts; u.P = P; u.window = window;
-  const int status = launch_lines<float, true>(nullptr, (const bf16_t*)W, (float*)C, M, N, heads * d, splits, s, u);
+  const int status = launch_lines<float, 1>(nullptr, (const bf16_t*)W, (float*)C, M, N, heads * d, splits, s, u);
+  if (status) return status;
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// 1 if qil_gemm_bf16_normed takes these sizes (rows, output columns, K, K splits).
+extern "C" int qil_gemm_bf16_normed_takes(int M, int N, int K, int splits) {
+  if (M < 1 || M > 16 || N < 1 || K % 8 || splits < 1 || K % (128 * splits) || K / (128 * splits) < LINES_DEPTH) return 0;
+  return lines_lds(M, K, splits) <= LINES_LDS_LIMIT;
+}
+
+// C float32 [splits, M, N] = partial sums of rmsnorm(stream; weight, eps) W^T, the norm made while the whole-line
+// kernel stages A from the float32 stream [M, K]; squares [pieces][M]: the rows' sums of squares in pieces.
+extern "C" int qil_gemm_bf16_normed(const float* stream, const float* weight, const float* squares, int pieces, float eps,
+                                    const void* W, void* C, int M, int N, int K, int splits, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  if (!qil_gemm_bf16_normed_takes(M, N, K, splits) || pieces < 1 ||
+      (((uintptr_t)W | (uintptr_t)stream | (uintptr_t)weight) % 16))
+    return -1;
+  NormedA n;
+  n.stream = stream; n.weight = weight; n.squares = squares; n.pieces = pieces; n.eps = eps;
+  const int status = launch_lines<float, 2>(nullptr, (const bf16_t*)W, (float*)C, M, N, K, splits, s, UnmergedA(), n);
   if (status) return status;
   QIL_RETURN_LAUNCH_STATUS();
 }

@@ -1,0 +1,194 @@
+// A few-row bfloat16 product that adds its result into the float32 residual stream:
+//   stream[M, N] += A[M, K] W[N, K]^T,   M <= 16, float32 accumulation.
+// A block owns `groups` groups of 16 output columns and `ksplit` waves per group, which split K among themselves and
+// add their float32 sums in LDS in wave order (the scheme of the gated kernel in gemm_bf16.hip): no partial sums in
+// memory, every element of the stream is read, added to and written by one lane, after its sum is complete.  The
+// kernel that follows finds the stream complete: it needs no sum over partial results, and the norm it would start
+// with can be made by the product after it (gemm_bf16.hip, NormedA), for which this kernel leaves the rows' sums of
+// squares in pieces: squares[piece][m] = sum over the 16 columns of group `piece` of stream[m, .]^2.
+// W and A both travel in whole cache lines (4 rows x 256 bytes a load), three stages of 128 columns ahead in
+// registers, through buffers of the wave's own in LDS that turn them into matrix-core fragments (see the whole-line
+// kernel in gemm_bf16.hip); A comes from L2.  K may be any length (the down product of a gated feed-forward).
+// Takes N a multiple of 16, K a multiple of 128 ksplit with at least 3 stages a wave, 16-byte aligned operands.
+#include <algorithm>
+
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define ADD_WAVES 8                                        // most waves of a block
+#define ADD_DEPTH 3                                        // stages in flight per wave
+#define ADD_LDS_LIMIT (160 * 1024)
+
+// AROWS: rows of A kept (8 or 16).
+template <int AROWS>
+__global__ void __launch_bounds__(ADD_WAVES * QIL_WAVE, AROWS == 8 ? 4 : 3)
+gemm_bf16_add_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, float* __restrict__ stream,
+                     float* __restrict__ squares, int M, int N, int K, int ksplit) {
+  extern __shared__ __align__(16) bf16_t lds[];            // per wave: 4 KB for W, AROWS x 256 bytes for A
+  constexpr int ALOADS = AROWS / 4, PER_WAVE = (16 + AROWS) * 128;
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int group = wave / ksplit, part = wave - group * ksplit;
+  const int groups = blockDim.x / QIL_WAVE / ksplit;
+  const int mine = blockIdx.x * groups + group;
+  const bool stores = mine * 16 < N;
+  const int n0 = min(mine, N / 16 - 1) * 16;               // a group past the end repeats the last one and stores nothing
+  const int cols = K / ksplit, k_begin = part * cols, stages = cols / 128;
+  // Every wave walks its K range from a start of its own and wraps around: waves that all read the same columns
+  // of their rows at the same time load a few memory channels only.
+  const int turn = (n0 / 16) % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * 128; };
+  bf16_t* buffer = lds + wave * PER_WAVE;
+  bf16_t* a_buffer = buffer + 16 * 128;
+
+  const int load_row = lane >> 4, piece = lane & 15;
+  const bf16_t* source[4];
+  const bf16_t* a_source[ALOADS];                          // rows past the last read it again: rows of D never stored
+  int place[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    source[u] = W + (size_t)(n0 + row) * K + k_begin + piece * 8;
+    place[u] = row * 128 + ((piece ^ row) & 15) * 8;
+    if (u < ALOADS) a_source[u] = A + (size_t)min(row, M - 1) * K + k_begin + piece * 8;
+  }
+  u32x4 w0[4], w1[4], w2[4], a0[ALOADS], a1[ALOADS], a2[ALOADS];   // named, so that none is indexed at run time
+  auto request = [&](u32x4 (&stage_w)[4], u32x4 (&stage_a)[ALOADS], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const u32x4*>(source[u] + at);
+#pragma unroll
+    for (int u = 0; u < ALOADS; ++u) stage_a[u] = *reinterpret_cast<const u32x4*>(a_source[u] + at);
+  };
+  request(w0, a0, 0);
+  request(w1, a1, 1);
+  request(w2, a2, 2);
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const int a_row = r & (AROWS - 1);
+  auto step = [&](u32x4 (&stage_w)[4], u32x4 (&stage_a)[ALOADS], int next, bool more) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x4*>(buffer + place[u]) = stage_w[u];
+#pragma unroll
+    for (int u = 0; u < ALOADS; ++u) *reinterpret_cast<u32x4*>(a_buffer + place[u]) = stage_a[u];
+    if (more) request(stage_w, stage_a, next);
+    __builtin_amdgcn_wave_barrier();                        // LDS operations of one wave complete in order: no wait
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      const u32x4 b = *reinterpret_cast<const u32x4*>(buffer + r * 128 + (((4 * s4 + kb) ^ r) & 15) * 8);
+      const u32x4 a = *reinterpret_cast<const u32x4*>(a_buffer + a_row * 128 + (((4 * s4 + kb) ^ a_row) & 15) * 8);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0,
+                                                    0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  int stage = 0;
+  for (; stage + 6 <= stages; stage += 3) {                 // every stage here has a successor three ahead
+    step(w0, a0, stage + 3, true);
+    step(w1, a1, stage + 4, true);
+    step(w2, a2, stage + 5, true);
+  }
+  const int left = stages - stage;                          // three to five stages: requests run out
+  step(w0, a0, stage + 3, left > 3);
+  step(w1, a1, stage + 4, left > 4);
+  step(w2, a2, 0, false);
+  if (left > 3) step(w0, a0, 0, false);
+  if (left > 4) step(w1, a1, 0, false);
+
+  // The waves' sums meet in LDS ([wave][lane][4] floats, in the buffers, which every wave has finished with); part 0 of
+  // each group adds them in wave order; the lane that holds D[m = 4 kb + i][n = r] adds it into the stream.
+  float* sums = reinterpret_cast<float*>(lds);
+  __syncthreads();
+  *reinterpret_cast<f32x4*>(sums + (wave * QIL_WAVE + lane) * 4) = acc;
+  __syncthreads();
+  if (part == 0) {
+    f32x4 total = {0.f, 0.f, 0.f, 0.f};
+    for (int v = wave; v < wave + ksplit; ++v)              // fixed order
+      total += *reinterpret_cast<const f32x4*>(sums + (v * QIL_WAVE + lane) * 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * kb + i;
+      float value = 0.f;
+      if (m < M && stores) {
+        float* cell = stream + (size_t)m * N + n0 + r;
+        value = *cell + total[i];
+        *cell = value;
+      }
+      if (squares) {                                        // the 16 lanes of a row add their squares: one order for all
+        float square = value * value;
+        square += __shfl_xor(square, 1, QIL_WAVE);
+        square += __shfl_xor(square, 2, QIL_WAVE);
+        square += __shfl_xor(square, 4, QIL_WAVE);
+        square += __shfl_xor(square, 8, QIL_WAVE);
+        if (r == 0 && m < M && stores) squares[(size_t)mine * M + m] = square;
+      }
+    }
+  }
+}
+
+static size_t add_lds_bytes(int M, int waves) {
+  return (size_t)waves * (16 + (M <= 8 ? 8 : 16)) * 128 * sizeof(bf16_t);     // also holds the waves' sums (1 KB a wave)
+}
+
+// Waves a group and groups a block for these sizes; false if the kernel does not take them.
+static bool add_plan(int M, int N, int K, int* groups, int* ksplit) {
+  if (M < 1 || M > 16 || N < 16 || N % 16 || K < 128 * ADD_DEPTH || K % 128) return false;
+  const int all_groups = N / 16;
+  int best_groups = 0, best_ksplit = 0;
+  double best_cost = 0;
+  for (int ks = 8; ks >= 1; ks /= 2) {
+    if (K % (128 * ks) || K / (128 * ks) < ADD_DEPTH) continue;
+    for (int gb = ADD_WAVES / ks; gb >= 1; --gb) {
+      const size_t lds = add_lds_bytes(M, gb * ks);
+      // blocks of a CU at a time: by LDS and by the wave slots its registers leave (16 for up to 8 rows, 12 beyond);
+      // rounds of the whole chip; a CU's waves keep memory busy when there are 8 or more of them
+      const long slots = M <= 8 ? 16 : 12;
+      const long together = std::max<long>(1, std::min<long>((long)(ADD_LDS_LIMIT / lds), slots / (gb * ks)));
+      const long blocks = (all_groups + gb - 1) / gb;
+      const long rounds = (blocks + 256 * together - 1) / (256 * together);
+      const long busy = std::min<long>(8, std::min<long>(together, (blocks + 255) / 256) * gb * ks);
+      const double cost = (double)rounds * gb * 8.0 / (double)busy + 0.05 * rounds;
+      if (!best_groups || cost < best_cost) { best_groups = gb; best_ksplit = ks; best_cost = cost; }
+    }
+  }
+  if (!best_groups) return false;
+  *groups = best_groups;
+  *ksplit = best_ksplit;
+  return true;
+}
+
+extern "C" {
+
+// 1 if qil_gemm_bf16_add takes these sizes.
+int qil_gemm_bf16_add_takes(int M, int N, int K) {
+  int groups, ksplit;
+  return add_plan(M, N, K, &groups, &ksplit);
+}
+
+// stream float32 [M, N] += A[M, K] W[N, K]^T.  squares: null, or float32 [N / 16][M] that gets the rows' sums of squares
+// of the new stream in pieces of 16 columns.  groups, ksplit: 0 = chosen here (tuning runs and tests set them).
+int qil_gemm_bf16_add(const void* A, const void* W, float* stream, float* squares, int M, int N, int K, int groups,
+                      int ksplit, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  if (((uintptr_t)A | (uintptr_t)W | (uintptr_t)stream) % 16) return -1;
+  int planned_groups, planned_ksplit;
+  if (!add_plan(M, N, K, &planned_groups, &planned_ksplit)) return -1;
+  if (!groups) groups = planned_groups;
+  if (!ksplit) ksplit = planned_ksplit;
+  if (groups < 1 || ksplit < 1 || groups * ksplit > ADD_WAVES || K % (128 * ksplit) || K / (128 * ksplit) < ADD_DEPTH)
+    return -1;
+  const size_t lds = add_lds_bytes(M, groups * ksplit);
+  dim3 grid((N / 16 + groups - 1) / groups), block(groups * ksplit * QIL_WAVE);
+  if (M <= 8)
+    hipLaunchKernelGGL(gemm_bf16_add_kernel<8>, grid, block, lds, s, (const bf16_t*)A, (const bf16_t*)W, stream, squares, M,
+                       N, K, ksplit);
+  else
+    hipLaunchKernelGGL(gemm_bf16_add_kernel<16>, grid, block, lds, s, (const bf16_t*)A, (const bf16_t*)W, stream, squares,
+                       M, N, K, ksplit);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -17,6 +17,7 @@ class Attention(Mixer):
     column is computed from the same row as before.
     """
     graph_safe = True
+    takes_lazy_norm = True       # h goes into ops.linear only, which takes a norm not computed yet
 
     def __init__(self, *, width, heads, kv_heads, head_dim, bias, qk_norm_eps, scale,
                  position=None, window=None, dtype=torch.bfloat16):

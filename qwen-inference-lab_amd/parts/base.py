@@ -72,6 +72,12 @@ class Norm(Part):
     def forward(self, stream, delta, out_dtype):
         raise NotImplementedError
 
+    def forward_lazy(self, stream, out_dtype, added):
+        """The norm of a stream that ``added`` (an ``ops.Added``) has just completed, as an object that a consumer's
+        kernel computes while it stages its operand (``ops.Normed``), or None where that does not apply.  Asked for
+        only by blocks whose consumer says it takes such an object (``takes_lazy_norm``)."""
+        return None
+
     def forward_rows(self, stream, delta, rows, out_dtype):
         raise NotImplementedError
 
@@ -109,6 +115,8 @@ class Mixer(Part):
     # be captured into a HIP graph and replayed with other contents.  A new graph runs its first step
     # once launch by launch and once more as the first replay.
     graph_safe = False
+    # True if forward takes ``h`` as an ``ops.Normed`` (a norm not computed yet) as well as a tensor.
+    takes_lazy_norm = False
 
     def cache_need(self):
         return None
@@ -118,7 +126,12 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Per-token map [N, width] -> [N, width] (tensor of the model's type or ``ops.Partials``)."""
+    """Per-token map [N, width] -> [N, width] (tensor of the model's type or ``ops.Partials``).
+
+    A part that sets ``adds_to_stream`` is called as ``forward(h, add_to=stream)`` and may add its result into
+    the float32 residual stream itself; it then returns the ``ops.Added`` that its last product gave."""
+    adds_to_stream = False
+
     def forward(self, h):
         raise NotImplementedError
 
@@ -129,7 +142,8 @@ class Block(Part):
     ``forward(stream, pending, ctx, cache)`` -> pending: ``stream`` is the float32
     residual stream [N, width], changed in place; ``pending`` is a sub-layer
     output not yet added to it (or None), which lets the add fuse into the next
-    norm.  The block returns its own last sub-layer output as the new pending.
+    norm.  The block returns its own last sub-layer output as the new pending; an
+    ``ops.Added`` says that the output is in the stream already.
     """
     mixer = None
 

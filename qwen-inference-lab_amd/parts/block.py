@@ -5,6 +5,7 @@ stream is float32 and every residual sum is made in float32; the add of a
 sub-layer's output is fused into the norm that follows it.
 """
 from .base import Block
+from .. import ops
 
 
 class PreNormBlock(Block):
@@ -19,7 +20,13 @@ class PreNormBlock(Block):
                 n['ffn_norm']: self.ffn_norm, n['ffn']: self.ffn}
 
     def forward(self, stream, pending, ctx, cache):
-        h = self.mixer_norm.forward(stream, pending, self.dtype)
+        h = None
+        if isinstance(pending, ops.Added):                     # the stream is complete
+            if self.mixer.takes_lazy_norm:                     # the mixer's first product may make the norm itself
+                h = self.mixer_norm.forward_lazy(stream, self.dtype, pending)
+            pending = None
+        if h is None:
+            h = self.mixer_norm.forward(stream, pending, self.dtype)
         mixed = self.mixer.forward(h, ctx, cache)
-        h = self.ffn_norm.forward(stream, mixed, self.dtype)
-        return self.ffn.forward(h)
+        h = self.ffn_norm.forward(stream, None if isinstance(mixed, ops.Added) else mixed, self.dtype)
+        return self.ffn.forward(h, add_to=stream) if self.ffn.adds_to_stream else self.ffn.forward(h)

@@ -26,6 +26,10 @@ class GatedMLP(FeedForward):
         p = self.p
         p['gate_up_proj.weight'] = torch.cat([p.pop('gate_proj.weight'), p.pop('up_proj.weight')]).contiguous()
 
-    def forward(self, h):
+    adds_to_stream = True
+
+    def forward(self, h, add_to=None):
         hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype)
+        if add_to is not None and hidden.is_cuda:              # few rows: the down product adds into the stream itself
+            return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True, add_to=add_to)
         return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

@@ -4,6 +4,7 @@ from dataclasses import dataclass
 import torch
 
 from .base import KVNeed, StateNeed
+from .. import ops
 
 
 @dataclass(frozen=True)
@@ -101,5 +102,7 @@ class CausalLM:
             pending = self.blocks[entry.block].forward(stream, pending, ctx, cache)
         if ctx.n_logit_rows == 0:
             return None
+        if isinstance(pending, ops.Added):                      # the last block's output is in the stream already
+            pending = None
         rows = self.final_norm.forward_rows(stream, pending, ctx.logit_rows, self.dtype)
         return self.head.forward(rows)

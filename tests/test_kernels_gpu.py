@@ -211,6 +211,71 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
     check(whole[:16], few.double(), torch.float32, scale=8)
 
 
+@pytest.mark.parametrize('m,n,k', [(8, 4096, 12288), (1, 4096, 12288), (16, 1024, 3072), (3, 2560, 9728), (8, 5120, 25600),
+                                   (9, 5120, 17408), (4, 64, 384), (8, 4096, 4096)])
+def test_linear_adds_into_the_stream(ops, monkeypatch, m, n, k):
+    """The product whose epilogue adds the complete sums into the float32 residual stream and leaves the rows' sums of
+    squares in pieces of 16 columns, against float64."""
+    lib = ops.library.load()
+    x = rand(m, k, dtype=torch.bfloat16)
+    w = rand(n, k, dtype=torch.bfloat16, seed=3, scale=k ** -0.5)
+    before = rand(m, n, scale=2.0, seed=7)
+    expected = before.double() + x.double() @ w.double().t()
+    stream = before.clone()
+    assert lib.qil_gemm_bf16_add_takes(m, n, k)
+    monkeypatch.setattr(ops, 'ADD_GEMM_FEW_ROWS', 0)                              # whatever the sizes: the adding kernel
+    added = ops.linear(x, w, None, partials=True, add_to=stream)
+    assert isinstance(added, ops.Added) and added.squares.shape == (n // 16, m)
+    torch.testing.assert_close(stream.double().cpu(), expected.cpu(), atol=2e-4, rtol=1e-4)
+    pieces = stream.double().square().reshape(m, n // 16, 16).sum(-1).t()
+    torch.testing.assert_close(added.squares.double().cpu(), pieces.cpu(), atol=1e-5, rtol=1e-5)
+    raw = torch.cuda.current_stream().cuda_stream
+    for groups, ksplit in ((1, 8), (2, 4), (1, 2), (3, 1), (8, 1)):
+        if k % (128 * ksplit) or k // (128 * ksplit) < 3:
+            continue
+        stream = before.clone()
+        assert lib.qil_gemm_bf16_add(x.data_ptr(), w.data_ptr(), stream.data_ptr(), None, m, n, k, groups, ksplit, raw) == 0
+        torch.testing.assert_close(stream.double().cpu(), expected.cpu(), atol=2e-4, rtol=1e-4)
+    # what the kernel does not take comes back as a result to be added by the caller
+    tall = rand(40, k, dtype=torch.bfloat16)
+    stream = rand(40, n, seed=9)
+    kept = stream.clone()
+    assert not isinstance(ops.linear(tall, w, None, partials=True, add_to=stream), ops.Added)
+    torch.testing.assert_close(stream, kept, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize('m,n,k', [(1, 6144, 4096), (8, 6144, 4096), (16, 6144, 4096), (3, 4096, 1024), (8, 10240, 5120),
+                                   (5, 6144, 2560), (2, 48, 384), (7, 272, 1152)])
+def test_linear_of_a_normed_stream(ops, monkeypatch, m, n, k):
+    """The product that makes the RMSNorm of the residual stream while it stages its operand, from the sums of squares
+    that the adding product left, against the norm kernel followed by the product of partial sums: the same
+    normalised bfloat16 values (up to one rounding of the statistics), the same sums."""
+    stream = rand(m, k, scale=3.0)
+    weight = (1 + 0.3 * rand(k, seed=2)).contiguous()
+    w = rand(n, k, dtype=torch.bfloat16, seed=3, scale=k ** -0.5)
+    # the stream as an adding product leaves it: complete, with its squares in pieces
+    half = rand(m, 384, dtype=torch.bfloat16, seed=11)
+    monkeypatch.setattr(ops, 'ADD_GEMM_FEW_ROWS', 0)
+    added = ops.linear(half, rand(k, 384, dtype=torch.bfloat16, seed=12, scale=0.05), None, partials=True, add_to=stream)
+    assert isinstance(added, ops.Added)
+    kept = stream.clone()
+    lazy = ops.Normed(stream, weight, 1e-6, torch.bfloat16, added)
+    got = ops.linear(lazy, w, None, partials=True)
+    assert isinstance(got, ops.Partials)
+    torch.testing.assert_close(stream, kept, atol=0, rtol=0)                      # the stream is read only
+    normalised = ops.add_rmsnorm(stream.clone(), None, weight, 1e-6, torch.bfloat16)
+    torch.testing.assert_close(lazy.materialize(), normalised, atol=0, rtol=0)
+    want = ops.linear(normalised, w, None, partials=True)
+    assert isinstance(want, ops.Partials) and want.splits == got.splits
+    # a sum of squares in another order may move the statistics by one rounding, and a normalised value with it
+    torch.testing.assert_close(got.tensor, want.tensor, atol=2e-3, rtol=1e-3)
+    expected = normalised.double() @ w.double().t()
+    torch.testing.assert_close(got.sum().double().cpu(), expected.cpu(), atol=2e-3, rtol=1e-3)
+    # with a bias the norm kernel runs first: the same values
+    biased = ops.linear(ops.Normed(stream, weight, 1e-6, torch.bfloat16, added), w, rand(n, seed=5), partials=True)
+    torch.testing.assert_close(biased.double().cpu(), (expected + rand(n, seed=5).double()).cpu(), atol=0.03, rtol=0.02)
+
+
 @pytest.mark.parametrize('dtype', DTYPES)
 def test_silu_mul(ops, dtype):
     for inner in (136, 132, 131):                          # eight, four and one element a thread

@@ -241,3 +241,59 @@ def test_a_long_context_in_bfloat16_at_0p6b_sizes(tmp_path):
         assert torch.isfinite(got).all()
         print(f'{r}: {len(places)} places up to {max(places)}, max abs error {(got - expected).abs().max():.2e}, largest logit {scale:.2f}')
         torch.testing.assert_close(got, expected, atol=0.015 * scale, rtol=0.02)
+
+
+FEW_ROWS = {
+    '0.6B': dict(MIXED_06B),
+    '8B': dict(MIXED_06B, hidden_size=4096, intermediate_size=12288, num_attention_heads=32, tie_word_embeddings=False),
+    '4B': dict(MIXED_06B, hidden_size=2560, intermediate_size=9728, num_attention_heads=32),
+    '32B': dict(MIXED_06B, hidden_size=5120, intermediate_size=25600, num_attention_heads=64, tie_word_embeddings=False),
+}
+
+
+@pytest.mark.parametrize('name,rows,always', [('0.6B', 3, False), ('0.6B', 11, False), ('8B', 12, False), ('8B', 5, True),
+                                              ('4B', 16, False), ('32B', 9, False)])
+def test_decode_steps_of_few_rows_at_real_sizes(tmp_path, monkeypatch, name, rows, always):
+    """Decode steps of 3 to 16 rows through two layers of real sizes in bfloat16: the down product adds into the
+    residual stream itself and the next layer's q/k/v product makes the norm from the sums of squares it left (with
+    ``always``: also where that is not the faster way).  Every logit against the plain model; replayed graphs against
+    launches."""
+    from qil_amd import ops
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.weights import load_model
+    from conftest import write_model_folder
+    config = FEW_ROWS[name]
+    weights = plain.random_weights(config, 17)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    model = load_model(folder, dtype=torch.bfloat16, device='cuda')
+    if always:
+        monkeypatch.setattr(ops, 'ADD_GEMM_FEW_ROWS', 0)
+    made = []
+    real = ops.Normed.__init__
+    monkeypatch.setattr(ops.Normed, '__init__', lambda self, *a, **k: (made.append(1), real(self, *a, **k))[1])
+    sequences = [random_tokens(config, 9 + (5 * i) % 23, 50 + i) for i in range(rows)]
+    new = 5
+    outputs = []
+    for with_graphs in (True, False):
+        runner = ModelRunner(model, num_pages=rows * 3, page_size=16, max_requests=rows, graphs=with_graphs)
+        poison(runner)
+        for r, tokens in enumerate(sequences):
+            runner.admit(r)
+        runner.step([StepEntry(r, tuple(tokens[:-new]), ()) for r, tokens in enumerate(sequences)])
+        made.clear()
+        steps = []
+        for k in range(new):
+            entries = [StepEntry(r, (tokens[len(tokens) - new + k],), (0,)) for r, tokens in enumerate(sequences)]
+            steps.append(runner.step(entries).cpu())
+        assert made, 'the q/k/v product of the second layer made its norm itself'
+        outputs.append(steps)
+    expected = [plain.logits(tokens, weights, config) for tokens in sequences]
+    worst = 0.0
+    for k in range(new):
+        want = torch.stack([expected[r][len(tokens) - new + k] for r, tokens in enumerate(sequences)])
+        scale = max(1.0, want.abs().max().item())
+        assert torch.isfinite(outputs[0][k]).all()
+        torch.testing.assert_close(outputs[0][k], outputs[1][k], atol=0.008 * scale, rtol=0.02)
+        torch.testing.assert_close(outputs[0][k], want, atol=0.015 * scale, rtol=0.02)
+        worst = max(worst, (outputs[0][k] - want).abs().max().item() / scale)
+    print(f'{name} {rows} rows: largest error {worst:.4f} of the largest logit')
