@@ -143,45 +143,53 @@ add_rmsnorm_vec_kernel(float* __restrict__ stream, const TD* __restrict__ delta,
   }
 }
 
-// out[n, i] = silu(gate_up[n, i]) * gate_up[n, inner + i], silu(z) = z * sigmoid(z)   (qil/model.py:71)
+// out[n, i] = silu(gate[n, i]) * up[n, i], silu(z) = z * sigmoid(z)   (qil/model.py:71).  The two halves of a row of
+// gate_up [n, 2 inner] are stacked (gate columns first: gate i at i, up i at inner + i) or interleaved in tiles of 16
+// columns (gate tile, up tile, gate tile, ...: gate i at 32 (i / 16) + i % 16, up i 16 further; inner % 16 == 0).
+__device__ __forceinline__ size_t gate_column(int i, int interleaved) {
+  return interleaved ? (size_t)(i >> 4) * 32 + (i & 15) : (size_t)i;
+}
 template <typename TD, typename T>
 __global__ void silu_mul_kernel(const TD* __restrict__ gate_up, int splits, size_t split_stride, T* __restrict__ out,
-                                int inner, size_t total) {
+                                int inner, size_t total, int interleaved) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t n = idx / inner;
   const int i = (int)(idx - n * inner);
-  const float g = load_sum(gate_up, n * 2 * (size_t)inner + i, splits, split_stride);
-  const float u = load_sum(gate_up, n * 2 * (size_t)inner + inner + i, splits, split_stride);
+  const size_t at = n * 2 * (size_t)inner + gate_column(i, interleaved);
+  const float g = load_sum(gate_up, at, splits, split_stride);
+  const float u = load_sum(gate_up, at + (interleaved ? 16 : inner), splits, split_stride);
   st(out + idx, (g / (1.f + expf(-g))) * u);
 }
 
 // Four outputs a thread, vector loads and stores; inner % 4 == 0.
 template <typename TD, typename T>
 __global__ void silu_mul_vec_kernel(const TD* __restrict__ gate_up, int splits, size_t split_stride,
-                                    T* __restrict__ out, int inner, size_t total4) {
+                                    T* __restrict__ out, int inner, size_t total4, int interleaved) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total4) return;
   const int per_row = inner / 4;
   const size_t n = idx / per_row;
   const int i = (int)(idx - n * per_row) * 4;
-  const float4 g = load_sum4(gate_up, n * 2 * (size_t)inner + i, splits, split_stride);
-  const float4 u = load_sum4(gate_up, n * 2 * (size_t)inner + inner + i, splits, split_stride);
+  const size_t at = n * 2 * (size_t)inner + gate_column(i, interleaved);
+  const float4 g = load_sum4(gate_up, at, splits, split_stride);
+  const float4 u = load_sum4(gate_up, at + (interleaved ? 16 : inner), splits, split_stride);
   store4(out + n * (size_t)inner + i, make_float4((g.x / (1.f + expf(-g.x))) * u.x, (g.y / (1.f + expf(-g.y))) * u.y,
                                                   (g.z / (1.f + expf(-g.z))) * u.z, (g.w / (1.f + expf(-g.w))) * u.w));
 }
 
 // bfloat16 in and out, eight outputs a thread: 16-byte loads and stores (inner % 8 == 0).
 __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int inner,
-                                       size_t total8) {
+                                       size_t total8, int interleaved) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total8) return;
   const int per_row = inner / 8;
   const size_t n = idx / per_row;
   const int i = (int)(idx - n * per_row) * 8;
   float g[8], u[8], y[8];
-  ld8(gate_up + n * 2 * (size_t)inner + i, g);
-  ld8(gate_up + n * 2 * (size_t)inner + inner + i, u);
+  const size_t at = n * 2 * (size_t)inner + gate_column(i, interleaved);
+  ld8(gate_up + at, g);
+  ld8(gate_up + at + (interleaved ? 16 : inner), u);
 #pragma unroll
   for (int e = 0; e < 8; ++e) y[e] = (g[e] / (1.f + expf(-g[e]))) * u[e];
   *reinterpret_cast<uint4*>(out + n * (size_t)inner + i) =
@@ -250,15 +258,15 @@ int qil_add_rmsnorm(float* stream, const void* delta, int delta_dtype, int split
 
 // gate_up: in_dtype QIL_BF16 [n, 2 inner] or QIL_F32 [splits][n][2 inner] partial sums.
 int qil_silu_mul(const void* gate_up, int in_dtype, int splits, void* out, int n, int inner, int out_dtype,
-                 hipStream_t s) {
+                 int interleaved, hipStream_t s) {
   const size_t total = (size_t)n * inner;
   if (total == 0) return 0;
-  if (splits < 1 || (in_dtype == QIL_BF16 && splits != 1)) return -1;
+  if (splits < 1 || (in_dtype == QIL_BF16 && splits != 1) || (interleaved && inner % 16)) return -1;
   const size_t stride = (size_t)n * 2 * inner;
   if (in_dtype == QIL_BF16 && out_dtype == QIL_BF16 && inner % 8 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0)) {
     const size_t work8 = total / 8;
     hipLaunchKernelGGL(silu_mul_bf16x8_kernel, dim3((unsigned)((work8 + 255) / 256)), dim3(256), 0, s,
-                       (const bf16_t*)gate_up, (bf16_t*)out, inner, work8);
+                       (const bf16_t*)gate_up, (bf16_t*)out, inner, work8, interleaved);
     QIL_RETURN_LAUNCH_STATUS();
   }
   const bool vec = inner % 4 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0);
@@ -268,10 +276,10 @@ int qil_silu_mul(const void* gate_up, int in_dtype, int splits, void* out, int n
   do {                                                                                                                \
     if (vec)                                                                                                          \
       hipLaunchKernelGGL((silu_mul_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)gate_up, splits,      \
-                         stride, (T*)out, inner, work);                                                               \
+                         stride, (T*)out, inner, work, interleaved);                                                  \
     else                                                                                                              \
       hipLaunchKernelGGL((silu_mul_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)gate_up, splits, stride,  \
-                         (T*)out, inner, total);                                                                      \
+                         (T*)out, inner, total, interleaved);                                                         \
   } while (0)
   if (out_dtype == QIL_F32) {
     if (in_dtype != QIL_F32) return -1;

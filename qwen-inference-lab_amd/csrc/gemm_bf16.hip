@@ -395,7 +395,14 @@ static int launch_lines(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, 
 #define CHUNK_ROW (128 + GEMM_LDS_PAD)
 #define CHUNKS_MOST_ROWS 192
 
-template <typename OUT, int MT>
+// GATED: W is the [N = 2 inner, K] matrix of a gated feed-forward with gate and up rows interleaved in tiles of 16
+// (gate rows 0-15, up rows 0-15, gate rows 16-31, ...), and C [M, inner] gets silu(A gate^T) * (A up^T)
+// (qil/model.py:71).  A block then owns 64 columns of `inner`, 128 consecutive rows of W: the even waves make gate
+// products, the odd waves the up products that belong to them; these hand their sums over in LDS and the even waves
+// store the activations.  K is not split: no partial sums in memory and no separate activation pass.  (With the gate
+// rows stacked before the up rows a block would read two regions a power of two apart at the same columns at the
+// same time, which loads a few memory channels only: 59 us against 45 for 64 rows at 8B sizes.)
+template <typename OUT, int MT, bool GATED = false>
 __global__ void __launch_bounds__(LINES_WAVES * QIL_WAVE)
 gemm_bf16_chunks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N,
                         int K, int cols_per_split) {
@@ -405,7 +412,9 @@ gemm_bf16_chunks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   static_assert(PIECES >= 1, "a stage of A has fewer pieces than the block has threads");
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
-  const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16, split = blockIdx.z;
+  const int split = blockIdx.z;
+  const int inner_n0 = (blockIdx.x * (LINES_WAVES / 2) + (wave >> 1)) * 16;  // GATED: the wave's column of the result
+  const int n0 = (blockIdx.x * LINES_WAVES + wave) * 16;
   const int k_begin = split * cols_per_split, stages = cols_per_split / 128;
   bf16_t* buffer = lds + 2 * SLOT + wave * (16 * 128);
 
@@ -499,6 +508,28 @@ gemm_bf16_chunks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   }
   if (s < stages) step(s, w0, a1, std::false_type());
   if (s + 1 < stages) step(s + 1, w1, a2, std::false_type());
+  if (GATED) {
+    // every step ends with a barrier: the slots of A are free.  [up wave][tile][lane][4] floats
+    float* handed = reinterpret_cast<float*>(lds);
+    if (wave & 1)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4*>(handed + (((wave >> 1) * MT + t) * QIL_WAVE + lane) * 4) = acc[t];
+    __syncthreads();
+    if (!(wave & 1)) {
+      const int inner = N / 2;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const f32x4 up = *reinterpret_cast<const f32x4*>(handed + (((wave >> 1) * MT + t) * QIL_WAVE + lane) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int m = t * 16 + 4 * kb + i, n = inner_n0 + r;
+          const float g = acc[t][i];
+          if (m < M && n < inner) store_out(C + (size_t)m * inner + n, (g / (1.f + expf(-g))) * up[i]);
+        }
+      }
+    }
+    return;
+  }
   OUT* out = C + (size_t)split * M * N;
 #pragma unroll
   for (int t = 0; t < MT; ++t)
@@ -525,35 +556,37 @@ static int chunks_splits(int N, int K) {
   return splits;
 }
 
-template <typename OUT, int MT>
+template <typename OUT, int MT, bool GATED = false>
 static int launch_chunks_tiles(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
   const size_t lds = ((size_t)2 * 16 * MT * CHUNK_ROW + (size_t)LINES_WAVES * 16 * 128) * sizeof(bf16_t);
-  auto kernel = gemm_bf16_chunks_kernel<OUT, MT>;
+  auto kernel = gemm_bf16_chunks_kernel<OUT, MT, GATED>;
   static size_t granted = 0;                              // per instantiation
   if (lds > 64 * 1024 && lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     granted = lds;
   }
-  dim3 grid((N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
+  // GATED: a block owns 64 columns of the result (N / 2 of them), else 128 of N
+  dim3 grid(GATED ? (N / 2 + 63) / 64 : (N + 16 * LINES_WAVES - 1) / (16 * LINES_WAVES), 1, splits);
   hipLaunchKernelGGL(kernel, grid, dim3(LINES_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
   return 0;
 }
 
-template <typename OUT>
+template <typename OUT, bool GATED = false>
 static int launch_chunks(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N, int K, int splits, hipStream_t s) {
-  if (M <= 32) return launch_chunks_tiles<OUT, 2>(A, W, C, M, N, K, splits, s);
-  if (M <= 64) return launch_chunks_tiles<OUT, 4>(A, W, C, M, N, K, splits, s);
-  if (M <= 96) return launch_chunks_tiles<OUT, 6>(A, W, C, M, N, K, splits, s);
-  if (M <= 128) return launch_chunks_tiles<OUT, 8>(A, W, C, M, N, K, splits, s);
-  if (M <= 160) return launch_chunks_tiles<OUT, 10>(A, W, C, M, N, K, splits, s);
-  return launch_chunks_tiles<OUT, 12>(A, W, C, M, N, K, splits, s);
+  if (M <= 32) return launch_chunks_tiles<OUT, 2, GATED>(A, W, C, M, N, K, splits, s);
+  if (M <= 64) return launch_chunks_tiles<OUT, 4, GATED>(A, W, C, M, N, K, splits, s);
+  if (M <= 96) return launch_chunks_tiles<OUT, 6, GATED>(A, W, C, M, N, K, splits, s);
+  if (M <= 128) return launch_chunks_tiles<OUT, 8, GATED>(A, W, C, M, N, K, splits, s);
+  if (M <= 160) return launch_chunks_tiles<OUT, 10, GATED>(A, W, C, M, N, K, splits, s);
+  return launch_chunks_tiles<OUT, 12, GATED>(A, W, C, M, N, K, splits, s);
 }
 
 // ---------------------------------------------------------------------------------------------------
 // Gate and up products of a gated feed-forward with the activation in the epilogue:
 //   out[m, n] = silu(A W[n]^T) * (A W[inner + n]^T),  n < inner        (qil/model.py:71)
-// W is the stacked [2 inner, K] matrix, gate rows first.  A "pair" is 16 gate rows and the 16 up rows
+// W is the [2 inner, K] matrix with the gate rows stacked before the up rows, or with both interleaved in tiles of
+// 16 rows (gate rows 0-15, up rows 0-15, gate rows 16-31, ...).  A "pair" is 16 gate rows and the 16 up rows
 // that belong to them.  A block owns `pairs` consecutive pairs and `ksplit` waves per pair, which split
 // K among themselves and add their float32 sums in LDS in wave order, so nothing but the finished
 // activations leaves the block: no partial sums in memory and no separate activation pass.  All of A
@@ -562,11 +595,13 @@ static int launch_chunks(const bf16_t* A, const bf16_t* W, OUT* C, int M, int N,
 // Takes M <= 16 (while A fits in LDS), inner a multiple of 16, K a multiple of 128 ksplit with at least 2 stages a wave,
 // 16-byte aligned operands.
 #define GATED_MAX_WAVES 12                                 // three waves a SIMD: 168 registers each
+#define GATED_ROWS_FEWEST_BLOCKS 128                       // of the 17-to-192-row kernel: see gated_rows_takes
+#define GATED_ROWS_MOST 64                                 // beyond, the product and a separate activation are faster
 
 template <typename OUT>
 __global__ void __launch_bounds__(GATED_MAX_WAVES * QIL_WAVE)
 gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ out, int M,
-                       int inner, int K, int ksplit) {
+                       int inner, int K, int ksplit, int interleaved) {
   extern __shared__ __align__(16) bf16_t lds[];            // A [8 or 16][K + pad], then a 4 KB buffer per wave
   const int a_rows = M <= 8 ? 8 : 16;                      // rows of A kept (8 or 16: a power of two)
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
@@ -588,10 +623,11 @@ gemm_bf16_gated_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ 
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int row = 4 * u + load_row;
-    gate_source[u] = W + (size_t)(n0 + row) * K + k_begin + piece * 8;
+    gate_source[u] = W + (size_t)((interleaved ? 2 * n0 : n0) + row) * K + k_begin + piece * 8;
     place[u] = row * 128 + ((piece ^ row) & 15) * 8;
   }
-  const size_t up_offset = (size_t)inner * K;
+  // the up rows of a pair: `inner` rows after its gate rows (stacked), or right after them (interleaved in tiles of 16)
+  const size_t up_offset = (size_t)(interleaved ? 16 : inner) * K;
   // Every wave walks its K range from a start of its own and wraps around: waves that all read the
   // same columns of their rows at the same time load a few memory channels only.
   const int turn = (n0 / 16) % stages;
@@ -729,16 +765,37 @@ static bool gated_plan(const void* A, const void* W, int M, int inner, int K, in
   return true;
 }
 
-extern "C" int qil_gemm_bf16_gated_takes(int M, int inner, int K) {
+// 17 to 64 rows of a matrix with interleaved rows: the kernel that passes A through LDS in stages, with the gate's
+// epilogue.  It cannot split K, so it needs enough blocks of 64 result columns to fill the chip (`fewest`: 0 = the
+// measured bound, tests pass 1).  Measured against the product followed by the activation kernel, 64 rows: 45.0
+// against 47.6 us at 8B sizes (192 blocks), 108 against 117 at 32B sizes (400), 29 against 31 at 4B sizes (152); with
+// 128 rows the fused kernel loses (74 against 55 at 8B sizes: its 8 row tiles leave a wave too few registers).
+static bool gated_rows_takes(const void* A, const void* W, int M, int inner, int K, int interleaved, int fewest) {
+  if (!interleaved || M <= 16 || M > GATED_ROWS_MOST || inner < 16 || inner % 16 || K % 128 || K / 128 < LINES_DEPTH ||
+      (((uintptr_t)A | (uintptr_t)W) % 16))
+    return false;
+  return (inner + 63) / 64 >= (fewest ? fewest : GATED_ROWS_FEWEST_BLOCKS);
+}
+
+extern "C" int qil_gemm_bf16_gated_takes(int M, int inner, int K, int interleaved) {
   int pairs, ksplit;
-  return gated_plan(nullptr, nullptr, M, inner, K, &pairs, &ksplit);
+  return gated_plan(nullptr, nullptr, M, inner, K, &pairs, &ksplit) ||
+         gated_rows_takes(nullptr, nullptr, M, inner, K, interleaved, 0);
 }
 
 // out [M, inner] of out_dtype = silu(A W[:inner]^T) * (A W[inner:]^T).  pairs, ksplit: 0 = chosen here
 // (tuning runs set them).
 extern "C" int qil_gemm_bf16_gated(const void* A, const void* W, void* out, int M, int inner, int K, int out_dtype,
-                                   int pairs, int ksplit, hipStream_t s) {
+                                   int pairs, int ksplit, int interleaved, hipStream_t s) {
   if (M == 0 || inner == 0) return 0;
+  if (M > 16) {                                              // pairs: the fewest blocks to accept (tests pass 1)
+    if (!gated_rows_takes(A, W, M, inner, K, interleaved, pairs)) return -1;
+    const int status = out_dtype == QIL_F32
+                           ? launch_chunks<float, true>((const bf16_t*)A, (const bf16_t*)W, (float*)out, M, 2 * inner, K, 1, s)
+                           : launch_chunks<bf16_t, true>((const bf16_t*)A, (const bf16_t*)W, (bf16_t*)out, M, 2 * inner, K, 1, s);
+    if (status) return status;
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   int planned_pairs, planned_ksplit;
   if (!gated_plan(A, W, M, inner, K, &planned_pairs, &planned_ksplit)) return -1;
   if (!pairs) pairs = planned_pairs;
@@ -757,7 +814,7 @@ extern "C" int qil_gemm_bf16_gated(const void* A, const void* W, void* out, int 
       if (e != hipSuccess) return (int)e;                                                                            \
       granted = lds;                                                                                                 \
     }                                                                                                                \
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)out, M, inner, K, ksplit); \
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)out, M, inner, K, ksplit, interleaved); \
   }
   if (out_dtype == QIL_F32) QIL_GATED_CASE(float) else QIL_GATED_CASE(bf16_t)
 #undef QIL_GATED_CASE

@@ -310,41 +310,52 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False, add_to=None):
     return out
 
 
-def gated_linear(x, weight, out_dtype=None):
-    """silu(x @ gate^T) * (x @ up^T) with ``weight`` the stacked [2 I, K] matrix, gate rows first -> [N, I].
+def interleave_gate_up(gate, up):
+    """The [2 I, K] matrix that ``gated_linear(..., interleaved=True)`` takes: gate and up rows in turns of 16
+    (gate rows 0-15, up rows 0-15, gate rows 16-31, ...).  A pure re-layout; I must be a multiple of 16."""
+    inner, k = gate.shape
+    if up.shape != gate.shape or inner % 16:
+        raise ValueError('interleave_gate_up: two [I, K] matrices with I a multiple of 16')
+    return torch.stack((gate.view(inner // 16, 16, k), up.view(inner // 16, 16, k)), dim=1).reshape(2 * inner, k).contiguous()
 
-    One kernel when the fused few-row kernel takes the sizes (bfloat16, at most 16 rows); otherwise the
-    product followed by ``silu_mul``.  Both add in float32 and round once."""
+
+def gated_linear(x, weight, out_dtype=None, interleaved=False):
+    """silu(x @ gate^T) * (x @ up^T) -> [N, I], with ``weight`` the [2 I, K] matrix of both: the gate rows stacked
+    before the up rows, or (``interleaved``) both in turns of 16 rows, which the kernels read faster.
+
+    One kernel when a fused kernel takes the sizes (bfloat16; up to 16 rows, or up to 64 rows of an interleaved
+    matrix large enough to fill the chip); otherwise the product followed by ``silu_mul``.  Both add in float32."""
     if isinstance(x, Normed):
         x = x.materialize()
     _require(x, 'x')
     _require(weight, 'weight', x.dtype)
     n, k = x.shape
     both = weight.shape[0]
-    if weight.shape[1] != k or both % 2:
+    if weight.shape[1] != k or both % 2 or (interleaved and both % 32):
         raise ValueError(f'gated_linear: x {tuple(x.shape)}, weight {tuple(weight.shape)}')
     out_dtype = out_dtype or x.dtype
     lib = library.load()
-    if x.dtype == torch.bfloat16 and n and lib.qil_gemm_bf16_gated_takes(n, both // 2, k):
+    if x.dtype == torch.bfloat16 and n and lib.qil_gemm_bf16_gated_takes(n, both // 2, k, int(interleaved)):
         out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
         _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
-                                       _stream()), 'gemm_bf16_gated')
+                                       int(interleaved), _stream()), 'gemm_bf16_gated')
         return out
-    return silu_mul(linear(x, weight, None, partials=True), out_dtype)
+    return silu_mul(linear(x, weight, None, partials=True), out_dtype, interleaved=interleaved)
 
 
-def silu_mul(gate_up, out_dtype=None):
-    """[N, 2 I] (gate columns first; tensor of the model's type or Partials) -> silu(gate) * up, [N, I]."""
+def silu_mul(gate_up, out_dtype=None, interleaved=False):
+    """[N, 2 I] (tensor of the model's type or Partials) -> silu(gate) * up, [N, I].  The gate columns come first, or
+    (``interleaved``) gate and up columns come in turns of 16."""
     n, both = gate_up.shape
-    if both % 2:
-        raise ValueError('silu_mul: needs an even number of columns')
+    if both % 2 or (interleaved and both % 32):
+        raise ValueError('silu_mul: needs an even number of columns (a multiple of 32 when they are interleaved)')
     out_dtype = out_dtype or (gate_up.dtype if not isinstance(gate_up, Partials) else None)
     if out_dtype is None:
         raise ValueError('silu_mul of Partials needs out_dtype')
     pointer, code, splits = _operand(gate_up, 'gate_up', out_dtype, (n, both))
     out = torch.empty((n, both // 2), dtype=out_dtype, device=gate_up.device)
-    _check(library.load().qil_silu_mul(pointer, code, splits, _ptr(out), n, both // 2, _code(out_dtype), _stream()),
-           'silu_mul')
+    _check(library.load().qil_silu_mul(pointer, code, splits, _ptr(out), n, both // 2, _code(out_dtype), int(interleaved),
+                                       _stream()), 'silu_mul')
     return out
 
 

@@ -139,7 +139,7 @@ def _declare(lib):
     p, i, f, z = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
     lib.qil_embed.argtypes = [p, p, p, i, i, i, p]
     lib.qil_add_rmsnorm.argtypes = [p, p, i, i, i, p, p, p, i, i, f, i, i, p]
-    lib.qil_silu_mul.argtypes = [p, i, i, p, i, i, i, p]
+    lib.qil_silu_mul.argtypes = [p, i, i, p, i, i, i, i, p]
     lib.qil_add_bias.argtypes = [p, p, i, i, i, p]
     lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, p]
     lib.qil_attn_rows_workspace.argtypes = [i, i, i, i]
@@ -172,8 +172,8 @@ def _declare(lib):
     lib.qil_gemm_bf16_unmerged.argtypes = [p, p, p, p, i, i, i, i, i, i, i, i, p]
     lib.qil_gemm_bf16_unmerged_takes.argtypes = [i, i, i, i, i]
     lib.qil_gemm_bf16_unmerged_takes.restype = i
-    lib.qil_gemm_bf16_gated.argtypes = [p, p, p, i, i, i, i, i, i, p]
-    lib.qil_gemm_bf16_gated_takes.argtypes = [i, i, i]
+    lib.qil_gemm_bf16_gated.argtypes = [p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_gemm_bf16_gated_takes.argtypes = [i, i, i, i]
     lib.qil_gemm_bf16_gated_takes.restype = i
     lib.qil_gemm_bf16_normed_takes.argtypes = [i, i, i, i]
     lib.qil_gemm_bf16_normed_takes.restype = i

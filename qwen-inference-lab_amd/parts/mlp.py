@@ -7,8 +7,8 @@ from .. import ops
 
 class GatedMLP(FeedForward):
     """``activation`` names the gate's function; 'silu' (z * sigmoid(z)) is the one
-    the kernels have.  Gate and up matrices are stacked at ``finalize`` into one
-    [2 * intermediate, width] matrix (gate rows first): a pure re-layout."""
+    the kernels have.  Gate and up matrices become one [2 * intermediate, width] matrix at
+    ``finalize`` (rows in turns of 16, or gate rows first where the sizes do not allow that): a pure re-layout."""
 
     def __init__(self, *, width, intermediate, activation='silu', dtype=torch.bfloat16):
         super().__init__()
@@ -24,12 +24,15 @@ class GatedMLP(FeedForward):
 
     def finalize(self):
         p = self.p
-        p['gate_up_proj.weight'] = torch.cat([p.pop('gate_proj.weight'), p.pop('up_proj.weight')]).contiguous()
+        gate, up = p.pop('gate_proj.weight'), p.pop('up_proj.weight')
+        # on the GPU, rows in turns of 16 where the sizes allow (the kernels read a gate tile and its up tile side by side)
+        self.interleaved = self.intermediate % 16 == 0 and gate.is_cuda
+        p['gate_up_proj.weight'] = ops.interleave_gate_up(gate, up) if self.interleaved else torch.cat([gate, up]).contiguous()
 
     adds_to_stream = True
 
     def forward(self, h, add_to=None):
-        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype)
+        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype, interleaved=self.interleaved)
         if add_to is not None and hidden.is_cuda:              # few rows: the down product adds into the stream itself
             return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True, add_to=add_to)
         return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

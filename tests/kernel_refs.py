@@ -46,17 +46,24 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False):
     return y.to(out_dtype or x.dtype)
 
 
-def gated_linear(x, weight, out_dtype=None):
+def _halves(gate_up, interleaved):
+    """(gate, up) columns of [N, 2 I]: stacked, or in turns of 16 columns."""
+    inner = gate_up.shape[1] // 2
+    if not interleaved:
+        return gate_up[:, :inner], gate_up[:, inner:]
+    tiles = gate_up.reshape(gate_up.shape[0], inner // 16, 2, 16)
+    return tiles[:, :, 0].reshape(-1, inner), tiles[:, :, 1].reshape(-1, inner)
+
+
+def gated_linear(x, weight, out_dtype=None, interleaved=False):
     y = x.to(torch.float32) @ weight.to(torch.float32).t()
-    inner = y.shape[1] // 2
-    g, u = y[:, :inner], y[:, inner:]
+    g, u = _halves(y, interleaved)
     return (g / (1 + torch.exp(-g)) * u).to(out_dtype or x.dtype)
 
 
-def silu_mul(gate_up, out_dtype=None):
+def silu_mul(gate_up, out_dtype=None, interleaved=False):
     gate_up = _value(gate_up)
-    inner = gate_up.shape[1] // 2
-    g, u = gate_up[:, :inner].to(torch.float32), gate_up[:, inner:].to(torch.float32)
+    g, u = (t.to(torch.float32) for t in _halves(gate_up, interleaved))
     return (g / (1 + torch.exp(-g)) * u).to(out_dtype or gate_up.dtype)
 
 

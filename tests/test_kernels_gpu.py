@@ -301,6 +301,49 @@ def test_gated_linear(ops, m, inner, k, dtype):
     got = ops.gated_linear(x, w)
     assert got.dtype == dtype and got.shape == (m, inner)
     check(got, want, dtype, scale=8)
+    if inner % 16 == 0:                                   # the same with the rows in turns of 16
+        turns = ops.interleave_gate_up(w[:inner].contiguous(), w[inner:].contiguous())
+        assert torch.equal(turns[:16], w[:16]) and torch.equal(turns[16:32], w[inner:inner + 16])
+        check(ops.gated_linear(x, turns, interleaved=True), want, dtype, scale=8)
+        y_turns = (x.double() @ turns.double().t()).to(dtype)
+        check(ops.silu_mul(y_turns, interleaved=True), ops.silu_mul((x.double() @ w.double().t()).to(dtype)), dtype, scale=0)
+
+
+@pytest.mark.parametrize('m', [17, 32, 33, 64, 65, 96, 100, 128, 129, 160, 161, 192])
+@pytest.mark.parametrize('inner,k', [(12288, 4096), (8192, 1024), (8208, 384), (80, 512)])
+def test_gated_linear_of_17_to_192_rows(ops, m, inner, k):
+    """The gate's epilogue in the kernel that passes A through LDS in stages: a block owns 64 result columns, four
+    waves make the gate products and four the up products.  Where the op takes the sizes by itself (enough blocks to
+    fill the chip) it is that kernel that runs; small results are forced through it here.  Against float64, and
+    against the product followed by the activation."""
+    lib = ops.library.load()
+    x = rand(m, k, dtype=torch.bfloat16)
+    stacked = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
+    y = x.double() @ stacked.double().t()
+    want = torch.nn.functional.silu(y[:, :inner]) * y[:, inner:]
+    w = ops.interleave_gate_up(stacked[:inner].contiguous(), stacked[inner:].contiguous())
+    assert bool(lib.qil_gemm_bf16_gated_takes(m, inner, k, 1)) == (inner >= 8192 and m <= 64)
+    assert not lib.qil_gemm_bf16_gated_takes(m, inner, k, 0)                     # stacked rows: the two kernels
+    raw = torch.cuda.current_stream().cuda_stream
+    assert lib.qil_gemm_bf16_gated(x.data_ptr(), stacked.data_ptr(), x.data_ptr(), m, inner, k, 1, 1, 0, 0, raw) == -1
+    for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
+        out = torch.full((m, inner), float('nan'), dtype=dtype, device='cuda')
+        status = lib.qil_gemm_bf16_gated(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, inner, k, code, 1, 0, 1, raw)
+        if m > 64:
+            assert status == -1                                                   # the op's fallback is the faster way
+            continue
+        assert status == 0
+        if dtype == torch.float32:                           # float32 sums of K products: their rounding goes with their size
+            assert torch.isfinite(out).all()
+            torch.testing.assert_close(out.double().cpu(), want.cpu(), atol=2e-6 * want.abs().max().item(), rtol=1e-4)
+        else:
+            check(out, want, dtype, scale=8)
+    got = ops.gated_linear(x, w, interleaved=True)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, inner)
+    check(got, want, torch.bfloat16, scale=8)
+    unfused = ops.silu_mul(ops.linear(x, w, None, partials=True), torch.bfloat16, interleaved=True)
+    torch.testing.assert_close(got.float(), unfused.float(), atol=0.05, rtol=0.02)
+    check(ops.gated_linear(x, stacked), want, torch.bfloat16, scale=8)
 
 
 def test_gated_linear_block_shapes(ops):
@@ -312,10 +355,14 @@ def test_gated_linear_block_shapes(ops):
     w = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
     y = x.double() @ w.double().t()
     want = torch.nn.functional.silu(y[:, :inner]) * y[:, inner:]
+    turns = ops.interleave_gate_up(w[:inner].contiguous(), w[inner:].contiguous())
     stream = torch.cuda.current_stream().cuda_stream
     for pairs, ksplit in ((1, 1), (3, 4), (12, 1), (1, 8), (2, 2), (5, 2), (6, 2)):
         out = torch.full((m, inner), float('nan'), dtype=torch.float32, device='cuda')
-        assert lib.qil_gemm_bf16_gated(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, inner, k, 0, pairs, ksplit, stream) == 0
+        assert lib.qil_gemm_bf16_gated(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, inner, k, 0, pairs, ksplit, 0, stream) == 0
+        check(out, want, torch.float32, scale=8)
+        out.fill_(float('nan'))
+        assert lib.qil_gemm_bf16_gated(x.data_ptr(), turns.data_ptr(), out.data_ptr(), m, inner, k, 0, pairs, ksplit, 1, stream) == 0
         check(out, want, torch.float32, scale=8)
 
 
