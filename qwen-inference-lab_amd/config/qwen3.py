@@ -5,7 +5,8 @@ Same keys, defaults and rejections as the reference's ``ModelConfig``
 ``rope_theta`` 1e6, ``attention_bias`` false, ``tie_word_embeddings`` true when
 absent, ``eos_token_id`` int | list | null; ``model_type`` must be ``qwen3``;
 scaled RoPE, sliding windows, non-full layer types and activations other than
-SiLU are refused.
+SiLU are refused.  ``torch_dtype`` is kept as information only: weights are
+converted to the dtype the caller asks for.
 """
 from dataclasses import dataclass, fields, asdict
 
@@ -31,6 +32,7 @@ class Qwen3Config:
     attention_bias: bool = False          # qil/config.py:20
     tie_word_embeddings: bool = True      # qil/config.py:21 (default when the key is absent)
     eos_token_id: int | list | None = None
+    torch_dtype: str | None = None        # what the checkpoint says it was saved in; the caller's dtype decides
 
     architecture = 'Qwen3ForCausalLM'
     model_type = 'qwen3'
@@ -52,6 +54,8 @@ class Qwen3Config:
             raise ConfigError('eos_token_id must be an integer, a list of integers or null')
         if isinstance(eos, list):
             object.__setattr__(self, 'eos_token_id', list(eos))
+        if self.torch_dtype is not None and not isinstance(self.torch_dtype, str):
+            raise ConfigError('torch_dtype must be a string or null')
 
     @property
     def eos_ids(self):

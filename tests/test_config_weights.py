@@ -33,10 +33,12 @@ def test_config_fields_defaults_and_rejections(tmp_path):
     assert (defaults.rms_norm_eps, defaults.rope_theta, defaults.attention_bias, defaults.tie_word_embeddings,
             defaults.eos_token_id) == (1e-6, 1e6, False, True, None)
     assert Qwen3Config.from_dict(defaults.to_dict()) == defaults
+    assert defaults.torch_dtype is None                                          # informational: kept, never acted on
+    assert Qwen3Config.from_dict(dict(minimal, torch_dtype='bfloat16')).to_dict()['torch_dtype'] == 'bfloat16'
     for patch in (dict(model_type='qwen3_moe'), dict(rope_scaling={'rope_type': 'linear'}),      # tests/qil/test_model.py:72-80
                   dict(use_sliding_window=True), dict(hidden_act='gelu'), dict(layer_types=['sliding_attention']),
                   dict(vocab_size=0), dict(head_dim=15), dict(num_key_value_heads=3), dict(rms_norm_eps=0.0),
-                  dict(rope_theta=float('inf')), dict(hidden_size=64.0), dict(attention_bias='no')):
+                  dict(rope_theta=float('inf')), dict(hidden_size=64.0), dict(attention_bias='no'), dict(torch_dtype=16)):
         with pytest.raises(ConfigError):
             Qwen3Config.from_dict(dict(plain.TINY_A, **patch))
     with pytest.raises(ConfigError, match='required'):
