@@ -1,6 +1,7 @@
 """The description of one step's batch, on the host and on the device."""
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
 
@@ -36,3 +37,30 @@ class StepContext:
     host_starts: list = field(default_factory=list)
     host_slots: list = field(default_factory=list)
     requests: list = field(default_factory=list)
+
+
+class StepPieces:
+    """The integer arrays that describe a step, by name, and where each lies once they are laid end to end into
+    the one int32 array that goes to the device.  Names: ``tokens``, ``positions``, ``row_seq``, ``cu_seqlens``,
+    ``starts``, ``slots``, ``logit_rows``, ``single_rows``, and per page group g ``tables<g>`` (the block tables,
+    row-major) and ``token_slots<g>`` (the cache slot of every new token)."""
+
+    def __init__(self):
+        self.names, self.arrays = [], []
+
+    def add(self, name, array):
+        if name in self.names:
+            raise ValueError(f'piece {name!r} twice')
+        self.names.append(name)
+        self.arrays.append(np.asarray(array))
+
+    def sizes(self):
+        return [len(a) for a in self.arrays]
+
+    def spans(self):
+        """name -> (first, one past the last) index in the flat array."""
+        ends = np.cumsum([0] + self.sizes()).tolist()
+        return {name: (ends[i], ends[i + 1]) for i, name in enumerate(self.names)}
+
+    def flat(self):
+        return np.concatenate(self.arrays).astype(np.int32)

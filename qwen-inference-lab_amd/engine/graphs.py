@@ -39,7 +39,8 @@ MAX_SEEN = 256        # shapes remembered as seen once
 
 class _Graph:
     def __init__(self, runner, entries, pieces, facts, bucket, sampler=None):
-        self.sizes = [len(p) for p in pieces]
+        self.sizes = pieces.sizes()
+        self.spans = pieces.spans()
         rows = len(entries)
         self.described = sum(self.sizes)
         total = self.described + (3 * rows if sampler is not None else 0)
@@ -47,7 +48,6 @@ class _Graph:
         self.meta = torch.zeros(total, dtype=torch.int32, device=device)
         self.staging = torch.zeros(total, dtype=torch.int32).pin_memory()
         self.copied = torch.cuda.Event()
-        self.offsets = np.cumsum([0] + self.sizes).tolist()
         self.widths = list(facts['widths'])
         self.written = [[(None, 0)] * rows for _ in self.widths]     # per page group and row: (table, entries uploaded)
         self.drawn = self.drawn_host = None
@@ -76,16 +76,13 @@ class _Graph:
                 gc.enable()
 
     def load(self, pieces, packed=None):
+        if pieces.sizes() != self.sizes:
+            raise RuntimeError('batch layout does not fit the captured graph')
         self.copied.synchronize()                           # the previous upload has left the staging buffer
         flat = self.staging.numpy()
-        at = 0
-        for piece, size in zip(pieces, self.sizes):
-            if len(piece) != size:
-                raise RuntimeError('batch layout does not fit the captured graph')
-            flat[at:at + size] = piece
-            at += size
+        flat[:self.described] = pieces.flat()
         if packed is not None:
-            flat[at:] = packed.reshape(-1)
+            flat[self.described:] = packed.reshape(-1)
         self.meta.copy_(self.staging, non_blocking=True)
         self.copied.record()
 
@@ -95,18 +92,19 @@ class _Graph:
         entries; a table is a list that only grows, apart from given-back entries that no kernel reads).
         Holds the pages of the new tokens.  Returns the requests' positions."""
         cache = runner.cache
-        ps, offsets = cache.page_size, self.offsets
+        ps, spans = cache.page_size, self.spans
         starts = [cache.computed[e.request] for e in entries]
         for entry, start in zip(entries, starts):
             cache.ensure(entry.request, start + 1)
         self.copied.synchronize()
         flat = self.staging.numpy()
-        flat[offsets[0]:offsets[1]] = [e.tokens[0] for e in entries]
-        flat[offsets[1]:offsets[2]] = starts                # positions
-        flat[offsets[4]:offsets[5]] = starts                # where the requests' rows begin
-        flat[offsets[5]:offsets[6]] = [cache.slots[e.request] for e in entries]
+        put = lambda name, values: flat.__setitem__(slice(*spans[name]), values)
+        put('tokens', [e.tokens[0] for e in entries])
+        put('positions', starts)
+        put('starts', starts)                               # where the requests' rows begin
+        put('slots', [cache.slots[e.request] for e in entries])
         for group, width in enumerate(self.widths):
-            tables_at, slots_at, written = offsets[8 + 2 * group], offsets[9 + 2 * group], self.written[group]
+            tables_at, slots_at, written = spans[f'tables{group}'][0], spans[f'token_slots{group}'][0], self.written[group]
             for row, (entry, start) in enumerate(zip(entries, starts)):
                 table = cache.table(group, entry.request)
                 count = len(table)

@@ -12,7 +12,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager
-from .batch import StepContext, StepEntry
+from .batch import StepContext, StepEntry, StepPieces
 from .graphs import DecodeGraphs
 
 
@@ -64,11 +64,7 @@ class ModelRunner:
                 raise ValueError(f'request {entry.request!r}: wanted places must index its tokens')
 
     def _describe(self, entries, table_width=None, validate=True):
-        """Pages, then the batch description as host arrays: (entries, pieces, facts).
-
-        pieces: int arrays in a fixed order (tokens, positions, row_seq, cu_seqlens, starts, state
-        slots, logit rows, single rows, then per page group its block tables and token slots).
-        """
+        """Pages, then the batch description as host arrays: (entries, pieces, facts); pieces: a ``StepPieces``."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(e[0], tuple(e[1]), tuple(e[2]) if len(e) > 2 else ())
                    for e in entries]
         if validate:
@@ -88,7 +84,10 @@ class ModelRunner:
         logit_rows = np.fromiter((cu[i] + w for i, e in enumerate(entries) for w in e.want), dtype=np.int64)
         slots = [cache.slots[e.request] for e in entries]
         single = cu[:-1][np.asarray(counts) == 1] if max(counts) > 1 else np.zeros(0, dtype=np.int64)
-        pieces = [tokens, positions, row_seq, cu, np.asarray(starts), np.asarray(slots), logit_rows, single]
+        pieces = StepPieces()
+        for name, array in (('tokens', tokens), ('positions', positions), ('row_seq', row_seq), ('cu_seqlens', cu),
+                            ('starts', starts), ('slots', slots), ('logit_rows', logit_rows), ('single_rows', single)):
+            pieces.add(name, array)
         widths = []
         for index, group in enumerate(cache.kv_groups):
             tables = [cache.table(index, e.request) for e in entries]
@@ -101,34 +100,34 @@ class ModelRunner:
                 raise RuntimeError('a new token falls into a page that was given back')
             table[table < 0] = 0          # given-back blocks lie outside every window; never read
             widths.append(width)
-            pieces += [table.reshape(-1), token_slots]
+            pieces.add(f'tables{index}', table.reshape(-1))
+            pieces.add(f'token_slots{index}', token_slots)
         facts = dict(n=n, s=s, starts=starts, counts=counts, slots=slots, cu=cu.tolist(), widths=widths,
                      max_context=int(max(st + c for st, c in zip(starts, counts))), n_logit_rows=len(logit_rows))
         return entries, pieces, facts
 
     def _context(self, entries, pieces, facts, device_flat, max_context=None):
         """StepContext and cache views over a device int32 array holding the pieces back to back."""
-        offsets = np.cumsum([0] + [len(p) for p in pieces])
-        part = lambda i: device_flat[offsets[i]:offsets[i + 1]]
+        spans = pieces.spans()
+        part = lambda name: device_flat[spans[name][0]:spans[name][1]]
         s, counts = facts['s'], facts['counts']
         ctx = StepContext(
-            n_tokens=facts['n'], n_seqs=s, n_logit_rows=facts['n_logit_rows'], token_ids=part(0), positions=part(1),
-            row_seq=part(2), cu_seqlens=part(3), seq_starts=part(4), seq_slots=part(5), logit_rows=part(6),
-            single_rows=part(7) if max(counts) > 1 else None, max_query=max(counts),
+            n_tokens=facts['n'], n_seqs=s, n_logit_rows=facts['n_logit_rows'], token_ids=part('tokens'),
+            positions=part('positions'), row_seq=part('row_seq'), cu_seqlens=part('cu_seqlens'), seq_starts=part('starts'),
+            seq_slots=part('slots'), logit_rows=part('logit_rows'),
+            single_rows=part('single_rows') if max(counts) > 1 else None, max_query=max(counts),
             max_context=max_context or facts['max_context'], host_cu_seqlens=facts['cu'], host_starts=facts['starts'],
             host_slots=facts['slots'], requests=[e.request for e in entries])
         for view in self.views:
             if view is not None and hasattr(view, 'block_tables'):
-                at = 8 + 2 * view.group
-                view.block_tables = part(at).view(s, facts['widths'][view.group])
-                view.slots = part(at + 1)
+                view.block_tables = part(f'tables{view.group}').view(s, facts['widths'][view.group])
+                view.slots = part(f'token_slots{view.group}')
         return ctx
 
     def prepare(self, entries):
         """Pages, then the batch description on the device.  Does not touch the cache contents."""
         entries, pieces, facts = self._describe(entries)
-        flat = np.concatenate(pieces).astype(np.int32)
-        return entries, self._context(entries, pieces, facts, torch.from_numpy(flat).to(self.model.device))
+        return entries, self._context(entries, pieces, facts, torch.from_numpy(pieces.flat()).to(self.model.device))
 
     @torch.inference_mode()
     def step(self, entries):

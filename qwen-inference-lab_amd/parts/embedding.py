@@ -16,6 +16,11 @@ class Embedding(Part):
     def forward(self, token_ids):
         return ops.embed(token_ids, self.p['weight'])
 
+    def forward_step(self, ctx):
+        """The float32 stream [N, width] of a step's rows.  What the model calls; an embedding that also needs
+        the rows' positions (learned absolute positions, say) finds them in ``ctx`` (engine/batch.py)."""
+        return self.forward(ctx.token_ids)
+
 
 class LMHead(Part):
     """float32 logits = rows @ weight^T, no bias (qil/model.py:134).

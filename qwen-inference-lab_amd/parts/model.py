@@ -96,7 +96,7 @@ class CausalLM:
         Rows are selected before the final norm; with no wanted row neither the
         norm nor the head runs (qil/model.py:130-134).
         """
-        stream = self.embedding.forward(ctx.token_ids)
+        stream = self.embedding.forward_step(ctx)
         pending = None
         for entry, cache in zip(self.schedule, caches):
             pending = self.blocks[entry.block].forward(stream, pending, ctx, cache)

@@ -518,6 +518,107 @@ def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
         torch.testing.assert_close(pieces[name].double().cpu(), wanted[name], atol=2e-5, rtol=2e-4)
 
 
+def test_toy_embedding_with_learned_positions_and_a_scale(tmp_path):
+    """An embedding that the framework does not have, defined here: token rows times a constant plus learned rows by
+    absolute position (no rotation in the attention).  It reads the step's positions from the context, so portions
+    and decoded tokens get the rows of their own places; whole against pieces against a float64 restatement."""
+    from dataclasses import dataclass
+    from safetensors.torch import load_file
+    from qil_amd import ops
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.parts import (Attention, GatedMLP, ParamSpec, RMSNorm, PreNormBlock, Embedding, LMHead, CausalLM,
+                               ScheduleEntry)
+    from qil_amd.registry import register_architecture
+    from qil_amd.weights import write_random_model, load_model
+
+    class PlacedEmbedding(Embedding):
+        def __init__(self, vocab, width, places, scale):
+            super().__init__(vocab, width)
+            self.places, self.scale = places, scale
+
+        def param_specs(self):
+            return dict(super().param_specs(), **{'places.weight': ParamSpec((self.places, self.width))})
+
+        def forward_step(self, ctx):
+            rows = ops.embed(ctx.token_ids, self.p['weight'])
+            return rows * self.scale + self.p['places.weight'][ctx.positions.long()].float()
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        layers: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        inner: int
+        scale: float
+        eps: float = 1e-5
+        max_position_embeddings: int = 96
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+        def to_dict(self):
+            return dict(self.__dict__, architectures=['ToyPlacedLM'], model_type='toy_placed')
+
+    def build(c, *, dtype, device):
+        embedding = PlacedEmbedding(c.vocab_size, c.hidden_size, c.max_position_embeddings, c.scale)
+        blocks = [PreNormBlock(mixer_norm=RMSNorm(c.hidden_size, c.eps),
+                               mixer=Attention(width=c.hidden_size, heads=c.heads, kv_heads=c.kv_heads, head_dim=c.head_dim,
+                                               bias=False, qk_norm_eps=c.eps, scale=c.head_dim ** -0.5, position=None,
+                                               dtype=dtype),
+                               ffn_norm=RMSNorm(c.hidden_size, c.eps),
+                               ffn=GatedMLP(width=c.hidden_size, intermediate=c.inner, dtype=dtype), dtype=dtype)
+                  for _ in range(c.layers)]
+        final_norm, head = RMSNorm(c.hidden_size, c.eps), LMHead(c.vocab_size, c.hidden_size, tied_to=embedding)
+        names = {'embed.weight': (embedding, 'weight'), 'embed.places': (embedding, 'places.weight'),
+                 'norm.weight': (final_norm, 'weight')}
+        for i, block in enumerate(blocks):
+            for prefix, part in block.parts().items():
+                for local in part.param_specs():
+                    names[f'layers.{i}.{prefix}.{local}'] = (part, local)
+        return CausalLM(config=c, embedding=embedding, blocks=blocks, schedule=[ScheduleEntry(i) for i in range(len(blocks))],
+                        final_norm=final_norm, head=head, names=names, dtype=dtype, device=device)
+
+    register_architecture('ToyPlacedLM', model_type='toy_placed', config_class=ToyConfig, build=build, replace=True)
+    data = dict(architectures=['ToyPlacedLM'], model_type='toy_placed', vocab_size=140, hidden_size=40, layers=2, heads=4,
+                kv_heads=2, head_dim=16, inner=64, scale=1.75)
+    folder = write_random_model(tmp_path / 'placed', data, seed=5, dtype=torch.float32)
+    w = {k: v.double() for k, v in load_file(str(folder / 'model.safetensors')).items()}
+    c = ToyConfig.from_dict(data)
+
+    def expected(tokens):
+        n = len(tokens)
+        x = w['embed.weight'][tokens] * c.scale + w['embed.places'][:n]
+        positions = torch.arange(n)
+        for i in range(c.layers):
+            pre = f'layers.{i}.'
+            h = plain.rms_norm(x, w[pre + 'mixer_norm.weight'], c.eps)
+            q = plain.rms_norm((h @ w[pre + 'mixer.q_proj.weight'].t()).view(n, c.heads, c.head_dim), w[pre + 'mixer.q_norm.weight'], c.eps)
+            k = plain.rms_norm((h @ w[pre + 'mixer.k_proj.weight'].t()).view(n, c.kv_heads, c.head_dim), w[pre + 'mixer.k_norm.weight'], c.eps)
+            v = (h @ w[pre + 'mixer.v_proj.weight'].t()).view(n, c.kv_heads, c.head_dim)
+            x = x + plain.attention(q, k, v, positions, c.head_dim ** -0.5).reshape(n, -1) @ w[pre + 'mixer.o_proj.weight'].t()
+            h = plain.rms_norm(x, w[pre + 'ffn_norm.weight'], c.eps)
+            x = x + plain.gated_mlp(h, w[pre + 'ffn.gate_proj.weight'], w[pre + 'ffn.up_proj.weight'], w[pre + 'ffn.down_proj.weight'])
+        return plain.rms_norm(x, w['norm.weight'], c.eps) @ w['embed.weight'].t()
+
+    tokens = prompts_for(data, [37], 4)[0]
+    wanted = expected(tokens)
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+    for cuts in ([37], [20, 2, 1, 1, 1, 12]):
+        runner = ModelRunner(model, num_pages=5, page_size=8, max_requests=1)
+        runner.admit('a')
+        got, at = [], 0
+        for size in cuts:
+            got.append(runner.step([StepEntry('a', tuple(tokens[at:at + size]), tuple(range(size)))]))
+            at += size
+        torch.testing.assert_close(torch.cat(got).double().cpu(), wanted, atol=2e-5, rtol=2e-4)
+    shifted = expected(tokens[1:])                          # the places matter: the same tokens one place earlier differ
+    assert not torch.allclose(shifted, wanted[1:], atol=1e-3)
+
+
 def test_serving_loop_under_random_arrivals(model_folder):
     """A few hundred requests of mixed lengths arrive at random, some are cancelled, some sample with a
     temperature, with so few pages that many wait: every request ends, every page comes back, and the greedy
