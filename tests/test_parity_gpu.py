@@ -297,3 +297,32 @@ def test_decode_steps_of_few_rows_at_real_sizes(tmp_path, monkeypatch, name, row
         torch.testing.assert_close(outputs[0][k], want, atol=0.015 * scale, rtol=0.02)
         worst = max(worst, (outputs[0][k] - want).abs().max().item() / scale)
     print(f'{name} {rows} rows: largest error {worst:.4f} of the largest logit')
+
+
+@pytest.mark.parametrize('count', [1, 4, 12])
+def test_few_requests_through_the_serving_loop_at_real_sizes(tmp_path, count):
+    """One, four or twelve requests generate together at Qwen3-0.6B layer sizes in bfloat16 through ``Engine``: decode
+    steps of that many rows replay a graph that holds the adding down product, the q/k/v product that makes its own
+    norm and the draw.  Every token is the plain sampler's choice on the plain logits, up to bfloat16's margin."""
+    from qil_amd import Engine
+    from qil_amd.weights import load_model
+    from conftest import write_model_folder
+    config = MIXED_06B
+    weights = plain.random_weights(config, 23)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    model = load_model(folder, dtype=torch.bfloat16, device='cuda')
+    prompts = [random_tokens(config, 4 + (9 * i) % 31, 70 + i) for i in range(count)]
+    pages = 4 * count
+    engine = Engine(model, num_pages=pages, page_size=16, token_budget=64 * count, prefill_chunk=64, max_active=count)
+    results = engine.generate(prompts, max_new_tokens=7, ignore_eos=True)
+    stats = engine.stats()
+    assert stats['graph_replays'] >= 4 and stats['drawn'] == 7 * count and stats['pages_in_use'] == [0]
+    engine.cache.check()
+    assert engine.cache.free_pages == [pages]
+    for prompt, result in zip(prompts, results):
+        assert result['state'] == 'completed' and len(result['token_ids']) == 7
+        logits = plain.logits(prompt + result['token_ids'], weights, config)
+        for index, token in enumerate(result['token_ids']):
+            row = logits[len(prompt) + index - 1]
+            assert row[token] >= row.max() - 0.1, (index, token, int(row.argmax()))
+    engine.close()
