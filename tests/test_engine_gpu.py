@@ -619,6 +619,112 @@ def test_toy_embedding_with_learned_positions_and_a_scale(tmp_path):
     assert not torch.allclose(shifted, wanted[1:], atol=1e-3)
 
 
+def test_toy_rotation_of_neighbouring_pairs(tmp_path):
+    """Another position encoding without a change to the kernels: a rotation of the pairs (2 i, 2 i + 1) instead of
+    (i, i + d / 2).  Scores do not change when the same permutation is applied to the dimensions of queries and keys,
+    so the toy attention below re-lays the rows of its q and k projections (and its norm weights) once at load time,
+    evens first, and the engine's rotation does the rest.  Against a float64 restatement that rotates neighbours."""
+    from dataclasses import dataclass
+    from safetensors.torch import load_file
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.parts import (Attention, GatedMLP, Rotary, RMSNorm, PreNormBlock, Embedding, LMHead, CausalLM, ScheduleEntry)
+    from qil_amd.registry import register_architecture
+    from qil_amd.weights import write_random_model, load_model
+
+    class NeighbourPairsAttention(Attention):
+        def finalize(self):
+            d = self.head_dim
+            order = torch.cat([torch.arange(0, d, 2), torch.arange(1, d, 2)])
+            for name, heads in (('q_proj.weight', self.heads), ('k_proj.weight', self.kv_heads)):
+                w = self.p[name]
+                rows = (torch.arange(heads)[:, None] * d + order[None, :]).reshape(-1).to(w.device)
+                self.p[name] = w[rows].contiguous()
+            for name in ('q_norm.weight', 'k_norm.weight'):
+                self.p[name] = self.p[name][order.to(self.p[name].device)].contiguous()
+            super().finalize()
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        layers: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        inner: int
+        theta: float = 300.0
+        eps: float = 1e-5
+        max_position_embeddings: int = 96
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+        def to_dict(self):
+            return dict(self.__dict__, architectures=['ToyNeighboursLM'], model_type='toy_neighbours')
+
+    def build(c, *, dtype, device):
+        embedding = Embedding(c.vocab_size, c.hidden_size)
+        position = Rotary(c.head_dim, c.theta, c.max_position_embeddings, device=device)
+        blocks = [PreNormBlock(mixer_norm=RMSNorm(c.hidden_size, c.eps),
+                               mixer=NeighbourPairsAttention(width=c.hidden_size, heads=c.heads, kv_heads=c.kv_heads,
+                                                             head_dim=c.head_dim, bias=False, qk_norm_eps=c.eps,
+                                                             scale=c.head_dim ** -0.5, position=position, dtype=dtype),
+                               ffn_norm=RMSNorm(c.hidden_size, c.eps),
+                               ffn=GatedMLP(width=c.hidden_size, intermediate=c.inner, dtype=dtype), dtype=dtype)
+                  for _ in range(c.layers)]
+        final_norm, head = RMSNorm(c.hidden_size, c.eps), LMHead(c.vocab_size, c.hidden_size)
+        names = {'embed.weight': (embedding, 'weight'), 'norm.weight': (final_norm, 'weight'), 'head.weight': (head, 'weight')}
+        for i, block in enumerate(blocks):
+            for prefix, part in block.parts().items():
+                for local in part.param_specs():
+                    names[f'layers.{i}.{prefix}.{local}'] = (part, local)
+        return CausalLM(config=c, embedding=embedding, blocks=blocks, schedule=[ScheduleEntry(i) for i in range(len(blocks))],
+                        final_norm=final_norm, head=head, names=names, dtype=dtype, device=device)
+
+    register_architecture('ToyNeighboursLM', model_type='toy_neighbours', config_class=ToyConfig, build=build, replace=True)
+    data = dict(architectures=['ToyNeighboursLM'], model_type='toy_neighbours', vocab_size=130, hidden_size=48, layers=2,
+                heads=6, kv_heads=2, head_dim=16, inner=80)
+    folder = write_random_model(tmp_path / 'neighbours', data, seed=8, dtype=torch.float32)
+    w = {k: v.double() for k, v in load_file(str(folder / 'model.safetensors')).items()}
+    c = ToyConfig.from_dict(data)
+
+    def expected(tokens):
+        n, d = len(tokens), c.head_dim
+        inv_freq = 1.0 / c.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d)
+        angles = (torch.arange(n, dtype=torch.float32)[:, None] * inv_freq).double()
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+
+        def rotate(t):                                       # [n, heads, d]: the pairs (2 i, 2 i + 1)
+            a, b = t[..., 0::2], t[..., 1::2]
+            return torch.stack([a * cos - b * sin, a * sin + b * cos], dim=-1).reshape(t.shape)
+        x = w['embed.weight'][tokens]
+        positions = torch.arange(n)
+        for i in range(c.layers):
+            pre = f'layers.{i}.'
+            h = plain.rms_norm(x, w[pre + 'mixer_norm.weight'], c.eps)
+            q = plain.rms_norm((h @ w[pre + 'mixer.q_proj.weight'].t()).view(n, c.heads, d), w[pre + 'mixer.q_norm.weight'], c.eps)
+            k = plain.rms_norm((h @ w[pre + 'mixer.k_proj.weight'].t()).view(n, c.kv_heads, d), w[pre + 'mixer.k_norm.weight'], c.eps)
+            v = (h @ w[pre + 'mixer.v_proj.weight'].t()).view(n, c.kv_heads, d)
+            mixed = plain.attention(rotate(q), rotate(k), v, positions, d ** -0.5).reshape(n, -1)
+            x = x + mixed @ w[pre + 'mixer.o_proj.weight'].t()
+            h = plain.rms_norm(x, w[pre + 'ffn_norm.weight'], c.eps)
+            x = x + plain.gated_mlp(h, w[pre + 'ffn.gate_proj.weight'], w[pre + 'ffn.up_proj.weight'], w[pre + 'ffn.down_proj.weight'])
+        return plain.rms_norm(x, w['norm.weight'], c.eps) @ w['head.weight'].t()
+
+    tokens = prompts_for(data, [41], 2)[0]
+    wanted = expected(tokens)
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+    for cuts in ([41], [30, 1, 1, 1, 8]):
+        runner = ModelRunner(model, num_pages=6, page_size=8, max_requests=1)
+        runner.admit('a')
+        got, at = [], 0
+        for size in cuts:
+            got.append(runner.step([StepEntry('a', tuple(tokens[at:at + size]), tuple(range(size)))]))
+            at += size
+        torch.testing.assert_close(torch.cat(got).double().cpu(), wanted, atol=2e-5, rtol=2e-4)
+
+
 def test_serving_loop_under_random_arrivals(model_folder):
     """A few hundred requests of mixed lengths arrive at random, some are cancelled, some sample with a
     temperature, with so few pages that many wait: every request ends, every page comes back, and the greedy
