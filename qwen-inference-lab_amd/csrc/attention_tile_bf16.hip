@@ -106,7 +106,10 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   const int first_page = first_tile >> ps_shift, last_page = (key_end - 1) >> ps_shift;
   {
     const int* table = block_tables + (size_t)seq * table_stride;
-    for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS_) pages[i] = table[first_page + i];
+    // as the page's place in the cache in units of 256 bytes (a page of one kv head is 1 KB or more; 32 bits reach 1 TB)
+    const uint32_t page_units = (uint32_t)kv_heads * page_size * D / 128;
+    for (int i = threadIdx.x; i <= last_page - first_page; i += FAST_THREADS_)
+      pages[i] = (int)((uint32_t)table[first_page + i] * page_units);
   }
 
   int my_row[RB], my_pos[RB];
@@ -172,68 +175,80 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
   }
 
   // What this thread stages of every tile: K vector it = 16 bytes of key idx / (D / 8), V^T vector it =
-  // 8 keys (one 16-byte piece of a page row) of dim idx % D.
+  // 8 keys (one 16-byte piece of a page row) of dim idx % D, idx = thread + it * threads.  A wave's 64 vectors of
+  // one `it` lie in one page (K: 512 / D consecutive keys, 1 KB in a row; V^T: 64 dims of one group of 8 keys), so
+  // the page and everything else that changes from tile to tile is computed once a wave, on the scalar unit, and a
+  // lane adds an offset that never changes.  Only the page is kept inside the sequence's needed pages: any place in
+  // such a page is memory of the cache, and what lies outside [key_begin, key_end) is zeroed when published.
   // Addresses: 64 bits for the page (a cache may hold more than 2^31 elements), 32 bits within it.
   uint4 k_reg[K_ITERS], v_reg[V_ITERS];
-  const size_t page_stride = (size_t)kv_heads * page_size * D;
-  const uint32_t k_head = (uint32_t)kvh * page_size * D, v_head = (uint32_t)kvh * D * page_size;
+  constexpr int K_WAVE_KEYS = 512 / D, K_IT_KEYS = FAST_THREADS_ * 8 / D;   // keys of a wave's / the block's vectors of one `it`
+  constexpr int V_WAVES_PER_GROUP = D / QIL_WAVE;                           // waves that share a group of 8 keys
+  static_assert(K_ITERS == V_ITERS, "K and V^T vectors of one `it` cover the same keys");
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int low_page = key_begin >> ps_shift;
+  // The wave's K vectors of `it` are the keys it * K_IT_KEYS + k_wave .. of the tile, its V^T vectors the 8 keys from
+  // it * K_IT_KEYS + v_wave on: both in the same page (k_wave / 8 == v_wave / 8, pages hold 8 keys or more).
+  const int k_wave = wave_s * K_WAVE_KEYS, v_wave = wave_s / V_WAVES_PER_GROUP * 8;
+  const char* k_head = reinterpret_cast<const char*>(k_cache + (size_t)kvh * page_size * D);
+  const char* v_head =
+      reinterpret_cast<const char*>(v_cache + ((size_t)kvh * D + (wave_s % V_WAVES_PER_GROUP) * QIL_WAVE) * page_size);
+  const uint32_t k_lane = lane * 16, v_lane = lane * page_size * 2;          // bytes
+  // Lane `it` looks the page of the vectors `it` up, one request ahead: `held` is in a register when it is needed.
+  const int held_key = min(lane, K_ITERS - 1) * K_IT_KEYS + k_wave;
+  auto look_up = [&](int k0) { return pages[min(max((k0 + held_key) >> ps_shift, low_page), last_page) - first_page]; };
+  int held = 0;
   auto request = [&](int k0) {                             // page_size is a power of two here: ps_shift >= 0
-    int k_page[K_ITERS], v_page[V_ITERS];
-    uint32_t k_at[K_ITERS], v_at[V_ITERS];
+    const int in_page = k0 & (page_size - 1);              // 0 unless a page holds more keys than a tile
 #pragma unroll
-    for (int it = 0; it < K_ITERS; ++it) {                   // all the table entries first, then all the loads
-      const int idx = threadIdx.x + it * FAST_THREADS_;
-      const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
-      const int key = min(max(k0 + kl, key_begin), key_end - 1);     // clamped onto a needed key; zeroed when published
-      k_page[it] = pages[(key >> ps_shift) - first_page];
-      k_at[it] = k_head + (uint32_t)(key & (page_size - 1)) * D + dv;
+    for (int it = 0; it < K_ITERS; ++it) {
+      const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
+      const uint32_t k_in = (uint32_t)(in_page + ((it * K_IT_KEYS + k_wave) & (page_size - 1))) * (D * 2);
+      const uint32_t v_in = (uint32_t)(in_page + ((it * K_IT_KEYS + v_wave) & (page_size - 1))) * 2;
+      k_reg[it] = *reinterpret_cast<const uint4*>(k_head + page_at + k_in + k_lane);
+      v_reg[it] = *reinterpret_cast<const uint4*>(v_head + page_at + v_in + v_lane);
     }
-#pragma unroll
-    for (int it = 0; it < V_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS_;
-      const int grp = idx / D, dim = idx % D;
-      const int key = min(max(k0 + grp * 8, key_begin & ~7), (key_end - 1) & ~7);
-      v_page[it] = pages[(key >> ps_shift) - first_page];
-      v_at[it] = v_head + (uint32_t)dim * page_size + (uint32_t)(key & (page_size - 1));
-    }
-#pragma unroll
-    for (int it = 0; it < K_ITERS; ++it)
-      k_reg[it] = *reinterpret_cast<const uint4*>(k_cache + (size_t)k_page[it] * page_stride + k_at[it]);
-#pragma unroll
-    for (int it = 0; it < V_ITERS; ++it)
-      v_reg[it] = *reinterpret_cast<const uint4*>(v_cache + (size_t)v_page[it] * page_stride + v_at[it]);
+    held = look_up(k0 + BK);
   };
   // Key kl of a tile (= 32 a + 8 b + 4 c + e) is row 4 b + e of score sub-tile 2 a + c: lane (r, kb) of the
   // score product then holds, in sub-tiles 2 a and 2 a + 1, the keys 32 a + 8 kb .. + 7.  (WIDE: key
   // 32 a + 16 s + 8 h + 4 j + e is row 16 s + 8 j + 4 h + e of 32-key tile a.)
-  auto publish = [&](int k0, bf16_t* tile) {
-    bf16_t* Ks = tile;
-    bf16_t* Vt = tile + BK * K_ROW;
-    const bool inside = k0 >= key_begin && k0 + BK <= key_end;        // no key of the tile needs zeroing
+  int k_to[K_ITERS], v_to[V_ITERS];                        // where this thread's vectors go in a tile, in elements
 #pragma unroll
-    for (int it = 0; it < K_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS_;
-      const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
-      const int key = k0 + kl;
-      const bool valid = inside || (key >= key_begin && key < key_end);
-      const int row = WIDE ? (kl >> 5) * 32 + ((kl >> 4) & 1) * 16 + ((kl >> 2) & 1) * 8 + ((kl >> 3) & 1) * 4 + (kl & 3)
-                           : ((kl >> 5) * 2 + ((kl >> 2) & 1)) * 16 + ((kl >> 3) & 3) * 4 + (kl & 3);
-      *reinterpret_cast<uint4*>(Ks + row * K_ROW + dv) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
+  for (int it = 0; it < K_ITERS; ++it) {
+    const int idx = threadIdx.x + it * FAST_THREADS_;
+    const int kl = idx / (D / 8), dv = (idx % (D / 8)) * 8;
+    const int row = WIDE ? (kl >> 5) * 32 + ((kl >> 4) & 1) * 16 + ((kl >> 2) & 1) * 8 + ((kl >> 3) & 1) * 4 + (kl & 3)
+                         : ((kl >> 5) * 2 + ((kl >> 2) & 1)) * 16 + ((kl >> 3) & 3) * 4 + (kl & 3);
+    k_to[it] = row * K_ROW + dv;
+  }
+#pragma unroll
+  for (int it = 0; it < V_ITERS; ++it) {
+    const int idx = threadIdx.x + it * FAST_THREADS_;
+    v_to[it] = BK * K_ROW + (idx % D) * V_ROW + (idx / D) * 8;
+  }
+  auto publish = [&](int k0, bf16_t* tile) {
+    if (k0 >= key_begin && k0 + BK <= key_end) {           // no key of the tile needs zeroing
+#pragma unroll
+      for (int it = 0; it < K_ITERS; ++it) *reinterpret_cast<uint4*>(tile + k_to[it]) = k_reg[it];
+#pragma unroll
+      for (int it = 0; it < V_ITERS; ++it) *reinterpret_cast<uint4*>(tile + v_to[it]) = v_reg[it];
+      return;
     }
 #pragma unroll
-    for (int it = 0; it < V_ITERS; ++it) {
-      const int idx = threadIdx.x + it * FAST_THREADS_;
-      const int grp = idx / D, dim = idx % D;
-      uint4 raw = v_reg[it];
-      if (!inside) {       // zero what lies outside [key_begin, key_end): never written, or someone else's
-        const int key = k0 + grp * 8;
-        uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    for (int it = 0; it < K_ITERS; ++it) {
+      const int key = k0 + (threadIdx.x + it * FAST_THREADS_) / (D / 8);
+      const bool valid = key >= key_begin && key < key_end;
+      *reinterpret_cast<uint4*>(tile + k_to[it]) = valid ? k_reg[it] : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (!(key + e >= key_begin && key + e < key_end)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
-        raw = make_uint4(w[0], w[1], w[2], w[3]);
-      }
-      *reinterpret_cast<uint4*>(Vt + dim * V_ROW + grp * 8) = raw;
+    for (int it = 0; it < V_ITERS; ++it) {   // zero what lies outside [key_begin, key_end): never written, or someone else's
+      const int key = k0 + (threadIdx.x + it * FAST_THREADS_) / D * 8;
+      uint32_t w[4] = {v_reg[it].x, v_reg[it].y, v_reg[it].z, v_reg[it].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (!(key + e >= key_begin && key + e < key_end)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+      *reinterpret_cast<uint4*>(tile + v_to[it]) = make_uint4(w[0], w[1], w[2], w[3]);
     }
   };
 
@@ -396,6 +411,7 @@ attn_tile_bf16_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* 
     }
   };
   __syncthreads();                                         // the table entries are in place
+  held = look_up(first_tile);
   request(first_tile);
   if (TWO) {
     publish(first_tile, tiles);
