@@ -1,0 +1,401 @@
+// Prompt attention over the paged cache for bfloat16 and head size 128: the rows of a portion of a prompt against
+// all keys they see (qil/model.py:59-66 is the formula), keys and values loaded from memory straight into LDS.
+//
+// A block is 4 or 8 waves; a wave owns 32 rows of one head as ONE tile of v_mfma_f32_32x32x16_bf16, the waves of a
+// block are the heads of a kv group (and with 8 waves two row tiles): they share the staged keys.  Per tile of 64
+// keys: S^T = K Q^T (16 products), softmax statistics in float32 registers, O^T += V^T P^T (16 products).
+//
+// A wave issues one instruction every four cycles and a product keeps the matrix core for 32, so what a tile costs
+// is the number of instructions it takes and how many of them stand between two products.  Hence:
+//  * global_load_lds_dwordx4: a wave's load puts 1 KB from memory into LDS without passing registers, no LDS write
+//    instruction and no staging registers.  The 64 lanes' 16-byte pieces land side by side, so the layout in LDS is
+//    made by the choice of what each lane loads:
+//      K tile  [64 rows][16 pieces]: a load is 4 consecutive keys (1 KB of a page), piece p of row r holds the
+//              dims 8 (p ^ (r & 15)) ..: the fragment reads of 32 rows at one dim offset then spread over all banks;
+//      V tile  [8 groups of 8 keys][128 dims][8 keys]: a load is 64 dims of one group (the cache keeps V^T in
+//              pages, so 8 keys of a dim are 16 bytes in a row); a fragment read is 32 lanes side by side.
+//  * everything of a load's address that changes from tile to tile is the same for the whole wave (the page, found
+//    one tile ahead by one lane per load, and the place in it) and is computed on the scalar unit;
+//  * the next tile's loads are issued between the score products;
+//  * two tiles in LDS, one barrier a tile: after it every wave's loads of this tile have landed and every wave has
+//    finished with the tile before, whose place the next loads take.
+// Keys outside [key_begin, key_end) of a tile (the sequence's end within a page, a window's edge) get score -inf by
+// the mask; their values are zeroed in LDS, for a page may hold anything there.
+#include <type_traits>
+
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define PROMPT_D 128
+#define PROMPT_BK 64                                       // keys per tile
+#define PROMPT_TILE_BYTES (2 * PROMPT_BK * PROMPT_D * 2)   // K and V of a tile: 32 KB
+#define PROMPT_TABLE_MAX 4096                              // block-table entries of a sequence kept in LDS
+
+// Row of the score tile that key kl of a tile takes: key 32 a + 16 s + 8 h + 4 j + e is row 32 a + 16 s + 8 j + 4 h + e,
+// so that a lane's 16 scores of a 32-key tile are 8 consecutive keys twice: the B operand of the value product.
+__device__ __forceinline__ int prompt_row(int kl) {
+  return (kl & ~15) + ((kl >> 2) & 1) * 8 + ((kl >> 3) & 1) * 4 + (kl & 3);
+}
+
+template <int WAVES>
+__global__ void __launch_bounds__(WAVES * QIL_WAVE, WAVES == 4 ? 2 : 1)
+attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                   const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
+                   const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
+                   int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift,
+                   float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P,
+                   int parts) {
+  constexpr int D = PROMPT_D, BK = PROMPT_BK, THREADS = WAVES * QIL_WAVE;
+  constexpr int WFRAGS = D / 16, WTILES = D / 32;
+  constexpr int LOADS = 16 / WAVES;                        // K loads a wave and tile, and as many V loads
+  extern __shared__ __align__(1024) unsigned char lds[];   // two tiles (K then V each), then the table entries
+  int* pages = reinterpret_cast<int*>(lds + 2 * PROMPT_TILE_BYTES);
+
+  // Which sequence, row tile and (kv head, head chunk) this block takes.  Blocks go to the 8 XCDs in turn, each
+  // with an L2 of its own: when 256 is a multiple of the number of (sequence, kv head, chunk) triples, block id
+  // takes triple id % triples, so that an XCD sees the keys and values of few kv heads (one, with one sequence
+  // and 8 of them) and its L2 holds them; and of the row tiles, consecutive groups of 256 blocks walk them in
+  // opposite directions, so that the two blocks a CU holds make one long and one short pass over the keys.
+  int across, seq = blockIdx.y, pair = blockIdx.z;
+  const int triples = gridDim.y * gridDim.z, tiles_x = gridDim.x;
+  if (256 % triples == 0) {
+    const int id = blockIdx.x + tiles_x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int triple = id % triples;
+    seq = triple % gridDim.y;
+    pair = triple / gridDim.y;
+    const int place = id / triples, span = 2 * (256 / triples), base = place / span * span;
+    const int size = min(span, tiles_x - base), idx = place - base, upper = (size + 1) / 2;
+    across = base + (idx < upper ? size - 1 - idx : idx - upper);
+  } else {
+    const int linear = tiles_x * (blockIdx.y + gridDim.y * blockIdx.z);
+    across = ((linear >> 8) & 1) ? (int)blockIdx.x : tiles_x - 1 - (int)blockIdx.x;
+  }
+  // parts > 1 (a few row tiles against a long context): grid.z also counts the parts of P keys, and a block
+  // leaves float32 partial results (the layout of the split-context row kernels) for the merge kernel
+  const int part = pair / (kv_heads * chunks);
+  pair -= part * (kv_heads * chunks);
+  const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
+  if (n < 2) return;
+  const int RT = WAVES / GH;
+  const int block_rows = 32 * RT;
+  const int tile_row0 = across * block_rows;
+  if (tile_row0 >= n) return;
+  const int kvh = pair / chunks, chunk = pair % chunks;
+  const int g = heads / kv_heads;
+  const int lane = threadIdx.x & (QIL_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / QIL_WAVE);
+  const int head_local = chunk * GH + wave % GH, row_group = wave / GH;
+  const int wave_row0 = tile_row0 + row_group * 32;
+  const bool wave_active = head_local < g && wave_row0 < n;
+  const int head = kvh * g + head_local;
+  const int start = seq_starts[seq];
+
+  const int rows_in_block = min(block_rows, n - tile_row0);
+  const int pos_first = start + tile_row0;
+  int key_end = pos_first + rows_in_block;                             // last position + 1
+  int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  if (parts > 1) {                                                     // P is a multiple of the tile's keys
+    key_begin = max(key_begin, part * P);
+    key_end = min(key_end, (part + 1) * P);
+    if (key_begin >= key_end) return;                                  // no row of the block sees a key of this part
+  }
+  const int first_tile = key_begin / BK * BK;
+
+  // Block-table entries of [first_tile, key_end) into LDS, as the page's place in the cache in units of 256 bytes
+  // (a page of one kv head is 2 KB or more; 32 bits reach 1 TB).
+  const int first_page = first_tile >> ps_shift, last_page = (key_end - 1) >> ps_shift;
+  {
+    const int* table = block_tables + (size_t)seq * table_stride;
+    const uint32_t page_units = (uint32_t)kv_heads * page_size * D / 128;
+    for (int i = threadIdx.x; i <= last_page - first_page; i += THREADS)
+      pages[i] = (int)((uint32_t)table[first_page + i] * page_units);
+  }
+
+  // The wave's rows: lane = (row lane % 32, half lane / 32).
+  //   S^T[key, row] = K Q^T:  A = K rows (LDS), B = Q[row][dims 16 ks + 8 half ..]
+  //     -> the lane's 16 scores of 32-key tile kt are the keys 32 kt + 16 (i / 8) + 8 half + i % 8
+  //   O^T[dim, row] = V^T P^T:  A = V^T[dim lane % 32][keys 16 u + 8 half ..] (one 16-byte LDS read), B = scores 8 (u % 2) ..
+  //     -> the lane holds O[row][dims 32 t + 8 j + 4 half + e].
+  const int l32 = lane & 31, half = lane >> 5;
+  const int my_row = wave_row0 + l32;
+  const bool row_valid = wave_active && my_row < n;
+  const int my_pos = row_valid ? start + my_row : -1;      // a row past the end sees no key
+  const int wave_last_pos = start + min(n, wave_row0 + 32) - 1;        // nothing beyond it is visible to this wave
+  bf16x8 qw[WFRAGS];
+  {
+    const bf16_t* qrow = q + (size_t)(q0 + (row_valid ? my_row : 0)) * q_stride + (size_t)(wave_active ? head : 0) * D;
+#pragma unroll
+    for (int ks = 0; ks < WFRAGS; ++ks) {
+      uint4 raw = make_uint4(0, 0, 0, 0);
+      if (row_valid) raw = *reinterpret_cast<const uint4*>(qrow + ks * 16 + half * 8);
+      qw[ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+  float row_m = -INFINITY, row_l = 0.f;
+  f32x16 ow[WTILES];
+#pragma unroll
+  for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ow[t][i] = 0.f;
+
+  // ---- loads.  Load j = it * WAVES + wave of a tile: K keys 4 j .. 4 j + 3 (rows prompt_row(4 j) .. + 3, 1 KB), and
+  // V^T of the 64 dims 64 (j % 2) .. of the 8 keys from 8 (j / 2) on: both in the page of key 4 j.
+  const int low_page = key_begin >> ps_shift;
+  const char* k_head = reinterpret_cast<const char*>(k_cache + (size_t)kvh * page_size * D);
+  const char* v_head = reinterpret_cast<const char*>(v_cache + ((size_t)kvh * D + (wave & 1) * 64) * page_size);
+  // lane = (key lane / 16 of the four, piece lane % 16): it loads the dims that piece lane % 16 of its row holds
+  const int swizzle = ((wave & 1) << 3 | ((wave >> 1) & 1) << 2) + (lane >> 4);      // row & 15 of this lane's rows
+  const uint32_t k_lane = (lane >> 4) * (D * 2) + (((lane & 15) ^ swizzle) << 4);
+  const uint32_t v_lane = lane * page_size * 2;
+  // Lane `it` looks the page of the loads `it` up, one tile ahead: `held` is in a register when it is needed.
+  const int held_key = (min(lane, LOADS - 1) * WAVES + wave) * 4;
+  auto look_up = [&](int k0) { return pages[min(max((k0 + held_key) >> ps_shift, low_page), last_page) - first_page]; };
+  int held = 0;
+  // One K or V load of tile k0 (in_page = k0 % page_size) into the tile at `to`.
+  auto load_k = [&](int in_page, int it, unsigned char* to) {
+    const int key = (it * WAVES + wave) * 4;
+    const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
+    const uint32_t in = (uint32_t)(in_page + (key & (page_size - 1))) * (D * 2);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_head + page_at + in + k_lane),
+                                     (__attribute__((address_space(3))) void*)(to + prompt_row(key) * (D * 2)), 16, 0, 0);
+  };
+  auto load_v = [&](int in_page, int it, unsigned char* to) {
+    const int j = it * WAVES + wave;
+    const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
+    const uint32_t in = (uint32_t)(in_page + ((j >> 1) * 8 & (page_size - 1))) * 2;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_head + page_at + in + v_lane),
+                                     (__attribute__((address_space(3))) void*)(to + BK * D * 2 + j * 1024), 16, 0, 0);
+  };
+  auto load_tile = [&](int k0, unsigned char* to) {        // any k0: the pages are kept inside the needed ones
+#pragma unroll
+    for (int it = 0; it < LOADS; ++it) {
+      load_k(k0 & (page_size - 1), it, to);
+      load_v(k0 & (page_size - 1), it, to);
+    }
+    held = look_up(k0 + BK);
+  };
+  // Values of keys outside [key_begin, key_end) of the tile at `tile` become zero (K needs none: the mask).
+  auto zero_values = [&](int k0, unsigned char* tile) {
+    for (int idx = threadIdx.x; idx < BK / 8 * D; idx += THREADS) {
+      const int key = k0 + idx / D * 8;
+      if (key >= key_begin && key + 8 <= key_end) continue;
+      uint4* cell = reinterpret_cast<uint4*>(tile + BK * D * 2) + idx;
+      const uint4 raw = *cell;
+      uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (!(key + e >= key_begin && key + e < key_end)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+      *cell = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  };
+
+  // ---- one tile's arithmetic, with the loads of the next tile (into `next`) among the score products.
+  const float c = scale * 1.44269504088896f;               // p = exp2((s - m) c): the scale enters in the exponent
+  const uint32_t k_read = l32 * (D * 2), k_piece = half ^ (l32 & 15);        // piece 2 ks + half of row l32 is at (2 ks) ^ k_piece
+  const uint32_t v_read = (half * D + l32) * 16;
+  auto attend = [&](int k0, const unsigned char* tile, unsigned char* next, bool masked) {
+    const unsigned char* Ks = tile + k_read;
+    const unsigned char* Vt = tile + BK * D * 2 + v_read;
+    auto k_fragment = [&](int kt, int ks) {
+      return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Ks + kt * 32 * D * 2 + (((2 * ks) ^ k_piece) << 4)));
+    };
+    constexpr int AHEAD = 2;                               // steps of 16 dims whose fragments are on their way
+    bf16x8 ka[WFRAGS][2];
+#pragma unroll
+    for (int ks = 0; ks < AHEAD; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) ka[ks][kt] = k_fragment(kt, ks);
+    f32x16 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+    const int in_page = (k0 + BK) & (page_size - 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < WFRAGS; ++ks) {
+      if (ks + AHEAD < WFRAGS) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) ka[ks + AHEAD][kt] = k_fragment(kt, ks + AHEAD);
+      }
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][0], qw[ks], s[0], 0, 0, 0);
+      if (ks < 2 * LOADS) {                                // one load of the next tile
+        if (ks & 1) load_v(in_page, ks >> 1, next);
+        else load_k(in_page, ks >> 1, next);
+      }
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][1], qw[ks], s[1], 0, 0, 0);
+      if (ks == 2 * LOADS - 1) held = look_up(k0 + 2 * BK);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (masked) {                                          // keys a row does not see get score -inf (probability 0)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = k0 + 32 * kt + 16 * (i >> 3) + 8 * half + (i & 7);
+          const bool visible = key <= my_pos && (window <= 0 || key > my_pos - window);
+          s[kt][i] = visible ? s[kt][i] : -INFINITY;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+    const float m_new = fmaxf(row_m, mx);
+    const float base = (m_new == -INFINITY) ? 0.f : m_new;                                // exp(-inf - 0) = 0
+    const float shift = -base * c;
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(fmaf(row_m, c, shift));
+    if (m_new != row_m) {                        // nothing to rescale while the maximum stands
+#pragma unroll
+      for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ow[t][i] *= alpha;
+    }
+    row_m = m_new;
+    // probabilities, 16 keys at a time (scores 8 (u % 2) .. of 32-key tile u / 2), packed as the B operands of the value
+    // products right away: the float32 values are not kept
+    float psum = 0.f;
+    bf16x8 pb[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int kt = u >> 1, st = u & 1;
+      uint32_t packed[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[kt][8 * st + 2 * e], c, shift));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[kt][8 * st + 2 * e + 1], c, shift));
+        psum += p0;
+        psum += p1;
+        packed[e] = pack_bf16(p0, p1);
+      }
+      pb[u] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+    }
+    row_l = row_l * alpha + psum;
+    asm volatile("" : "+v"(row_l));                        // summed here, not after the products below
+    auto v_fragment = [&](int u, int t) {
+      return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Vt + u * (2 * D * 16) + t * (32 * 16)));
+    };
+    bf16x8 va[4][WTILES];
+#pragma unroll
+    for (int t = 0; t < WTILES; ++t) va[0][t] = v_fragment(0, t);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (u + 1 < 4) {
+#pragma unroll
+        for (int t = 0; t < WTILES; ++t) va[u + 1][t] = v_fragment(u + 1, t);
+      }
+#pragma unroll
+      for (int t = 0; t < WTILES; ++t) ow[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[u][t], pb[u], ow[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  __syncthreads();                                         // the table entries are in place
+  held = look_up(first_tile);
+  load_tile(first_tile, lds);
+  int buffer = 0;
+  for (int k0 = first_tile; k0 < key_end; k0 += BK, buffer ^= 1) {
+    unsigned char* tile = lds + buffer * PROMPT_TILE_BYTES;
+    unsigned char* next = lds + (buffer ^ 1) * PROMPT_TILE_BYTES;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's loads of the tile have landed
+    __syncthreads();                                       // everyone's have, and everyone is done with the tile before
+    if (!(k0 >= key_begin && k0 + BK <= key_end)) {
+      zero_values(k0, tile);
+      __syncthreads();
+    }
+    if (wave_active && k0 <= wave_last_pos) {
+      const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 32 <= n &&
+                               (window <= 0 || k0 > wave_last_pos - window);
+      attend(k0, tile, next, !all_visible);
+    } else {
+      load_tile(k0 + BK, next);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // no load into LDS is on its way when the block ends
+
+  if (!wave_active) return;
+  const float total = row_l + __shfl_xor(row_l, 32, QIL_WAVE);
+  if (!row_valid) return;
+  if (parts > 1) {
+    // acc [row, head, part, d] unnormalised, m (the maximum in the exponent's units) and l [row, head, part]; a row
+    // that sees no key of this part leaves m = -inf, l = 0 in a cell the merge does not read
+    const size_t cell = ((size_t)(q0 + my_row) * heads + head) * parts + part;
+#pragma unroll
+    for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<float4*>(part_acc + cell * D + 32 * t + 8 * j + 4 * half) =
+            make_float4(ow[t][4 * j], ow[t][4 * j + 1], ow[t][4 * j + 2], ow[t][4 * j + 3]);
+    if (half == 0) {
+      part_m[cell] = row_m == -INFINITY ? -INFINITY : row_m * scale;
+      part_l[cell] = total;
+    }
+    return;
+  }
+  const float inv = 1.f / total;
+  bf16_t* orow = out + ((size_t)(q0 + my_row) * heads + head) * D;
+#pragma unroll
+  for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)                             // dims 32 t + 8 j + 4 half + e, e < 4: 8 bytes
+      *reinterpret_cast<uint2*>(orow + 32 * t + 8 * j + 4 * half) =
+          make_uint2(pack_bf16(ow[t][4 * j] * inv, ow[t][4 * j + 1] * inv), pack_bf16(ow[t][4 * j + 2] * inv, ow[t][4 * j + 3] * inv));
+}
+
+template <int WAVES>
+static int launch_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                         int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
+                         int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s,
+                         float* workspace, int total_rows, int P, int parts) {
+  const int g = heads / kv_heads;
+  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = WAVES / GH;
+  const size_t lds = 2 * (size_t)PROMPT_TILE_BYTES + (size_t)table_stride * sizeof(int);
+  auto kernel = attn_prompt_kernel<WAVES>;
+  static size_t granted = 0;                     // per instantiation
+  if (lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((max_query + 32 * RT - 1) / (32 * RT), n_seqs, kv_heads * chunks * parts);
+  float* part_m = workspace ? workspace + (size_t)total_rows * heads * parts * PROMPT_D : nullptr;
+  float* part_l = part_m ? part_m + (size_t)total_rows * heads * parts : nullptr;
+  int ps_shift = -1;                                      // log2 of a power-of-two page size
+  for (int b = 0; b < 30; ++b)
+    if (page_size == (1 << b)) ps_shift = b;
+  hipLaunchKernelGGL(kernel, grid, dim3(WAVES * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+                     (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
+                     kv_heads, page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts);
+  return (int)hipGetLastError();
+}
+
+// 1 if the kernel of this file takes the sizes (bfloat16 only): head size 128, a page size that is a power of two
+// from 8 on, a block table of a sequence that fits in LDS beside two tiles.
+extern "C" int qil_attn_prompt_takes(int d, int page_size, int table_stride) {
+  return d == PROMPT_D && page_size >= 8 && (page_size & (page_size - 1)) == 0 && table_stride >= 1 &&
+         table_stride <= PROMPT_TABLE_MAX;
+}
+
+// Sequences with two or more rows (the others' rows stay unwritten).  waves: 4 or 8 a block.  parts == 1: out
+// [rows, heads * 128]; parts > 1: the keys in parts of P keys (a multiple of 64), float32 partial results in
+// `workspace` for the merge kernel, `out` unused.  The caller has checked the sizes (qil_attn_prompt_takes).
+extern "C" int qil_attn_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                               const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
+                               void* out, int n_seqs, int max_query, int heads, int kv_heads, int page_size, int window,
+                               float scale, int waves, void* workspace, int total_rows, int P, int parts, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if (!qil_attn_prompt_takes(PROMPT_D, page_size, table_stride) || heads % kv_heads || n_seqs > 65535 ||
+      (long)kv_heads * 2 * parts > 65535 || (waves != 4 && waves != 8) || parts < 1 ||
+      (parts > 1 && (!workspace || total_rows < 1 || P < PROMPT_BK || P % PROMPT_BK)) || (parts == 1 && !out))
+    return -1;
+  if (waves == 8)
+    return launch_prompt<8>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
+                            max_query, heads, kv_heads, page_size, window, scale, s, (float*)workspace, total_rows, P, parts);
+  return launch_prompt<4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
+                          max_query, heads, kv_heads, page_size, window, scale, s, (float*)workspace, total_rows, P, parts);
+}

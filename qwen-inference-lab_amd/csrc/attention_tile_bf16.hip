@@ -510,6 +510,12 @@ static int launch_fast(const void* q, int q_stride, const void* k_cache, const v
   return (int)hipGetLastError();
 }
 
+// The kernel for head size 128 (attention_prompt.hip).
+extern "C" int qil_attn_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                               const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
+                               void* out, int n_seqs, int max_query, int heads, int kv_heads, int page_size, int window,
+                               float scale, int waves, void* workspace, int total_rows, int P, int parts, hipStream_t s);
+
 static int tile_waves_override = 0;                       // tuning runs and tests: 4 or 8 forces the block size
 extern "C" void qil_attn_tile_waves(int waves) { tile_waves_override = waves; }
 
@@ -531,19 +537,16 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
   if (d == 64)
     return launch_fast<64, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
-  // Head size 128: blocks of 8 waves (64 rows of 4 heads, or 128 of 2, ... share a staged tile of keys; one block
-  // a CU) once blocks of 4 waves would be four or more a CU: measured equal at 4 x 1024 tokens of 32 heads,
-  // 5 % faster at 4,096 tokens, 18 % at 8,192, and slower below (2,048 tokens: 81 against 80 us).
-  const int g128 = heads / kv_heads, gh128 = g128 >= 3 ? 4 : g128;
-  const long blocks4 = (long)((max_query + 32 * (4 / gh128) - 1) / (32 * (4 / gh128))) * n_seqs * kv_heads *
-                       ((g128 + gh128 - 1) / gh128);
-  const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 1024;
-  if (d == 128 && wide)
-    return launch_fast<128, 2, 8>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
-                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
-  if (d == 128)
-    return launch_fast<128, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
-                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
+  // Head size 128 has a kernel of its own (attention_prompt.hip).  Blocks of 8 waves (64 rows of 4 heads, or 128 of
+  // 2, ... share a staged tile of keys; one block a CU) once blocks of 4 waves would be four or more a CU.
+  if (d == 128) {
+    const int g128 = heads / kv_heads, gh128 = g128 >= 3 ? 4 : g128;
+    const long blocks4 = (long)((max_query + 32 * (4 / gh128) - 1) / (32 * (4 / gh128))) * n_seqs * kv_heads *
+                         ((g128 + gh128 - 1) / gh128);
+    const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 1024;
+    return qil_attn_prompt(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
+                           max_query, heads, kv_heads, page_size, window, scale, wide ? 8 : 4, nullptr, 0, 0, 1, s);
+  }
   return launch_fast<256, 1, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                 n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
 }
@@ -587,7 +590,7 @@ extern "C" int qil_attn_tile_bf16_parts(const void* q, int q_stride, const void*
     return launch_fast<64, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
                                  nullptr, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
                                  (float*)workspace, total_rows, P, parts);
-  return launch_fast<128, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
-                                nullptr, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
-                                (float*)workspace, total_rows, P, parts);
+  return qil_attn_prompt(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, nullptr,
+                         n_seqs, max_query, heads, kv_heads, page_size, window, scale, 4, workspace, total_rows, P, parts,
+                         s);
 }
