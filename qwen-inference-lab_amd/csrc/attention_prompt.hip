@@ -18,7 +18,12 @@
 //    one tile ahead by one lane per load, and the place in it) and is computed on the scalar unit;
 //  * the next tile's loads are issued between the score products;
 //  * two tiles in LDS, one barrier a tile: after it every wave's loads of this tile have landed and every wave has
-//    finished with the tile before, whose place the next loads take.
+//    finished with the tile before, whose place the next loads take;
+//  * the reference of a row's exponents is only moved (to the maximum) when a score exceeds it by 2^8 in the
+//    exponent: the sums then hold probabilities up to 2^8 instead of 1, which float32 and bfloat16 bear, and the 64
+//    multiplications that rescale a wave's results become rare;
+//  * only a block's first and last tile can hold keys outside [key_begin, key_end): the loop over the tiles between
+//    has no code for that case (its presence alone, never run, cost a tenth of the loop's time).
 // Keys outside [key_begin, key_end) of a tile (the sequence's end within a page, a window's edge) get score -inf by
 // the mask; their values are zeroed in LDS, for a page may hold anything there.
 #include <type_traits>
@@ -151,24 +156,27 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   const uint32_t v_lane = lane * page_size * 2;
   // Lane `it` looks the page of the loads `it` up, one tile ahead: `held` is in a register when it is needed.
   const int held_key = (min(lane, LOADS - 1) * WAVES + wave) * 4;
-  auto look_up = [&](int k0) { return pages[min(max((k0 + held_key) >> ps_shift, low_page), last_page) - first_page]; };
+  auto look_up = [&](int k0) __attribute__((always_inline)) {
+    return pages[min(max((k0 + held_key) >> ps_shift, low_page), last_page) - first_page];
+  };
   int held = 0;
   // One K or V load of tile k0 (in_page = k0 % page_size) into the tile at `to`.
-  auto load_k = [&](int in_page, int it, unsigned char* to) {
+  auto load_k = [&](int in_page, int it, unsigned char* to) __attribute__((always_inline)) {
     const int key = (it * WAVES + wave) * 4;
     const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
     const uint32_t in = (uint32_t)(in_page + (key & (page_size - 1))) * (D * 2);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_head + page_at + in + k_lane),
                                      (__attribute__((address_space(3))) void*)(to + prompt_row(key) * (D * 2)), 16, 0, 0);
   };
-  auto load_v = [&](int in_page, int it, unsigned char* to) {
+  auto load_v = [&](int in_page, int it, unsigned char* to) __attribute__((always_inline)) {
     const int j = it * WAVES + wave;
     const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
     const uint32_t in = (uint32_t)(in_page + ((j >> 1) * 8 & (page_size - 1))) * 2;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_head + page_at + in + v_lane),
                                      (__attribute__((address_space(3))) void*)(to + BK * D * 2 + j * 1024), 16, 0, 0);
   };
-  auto load_tile = [&](int k0, unsigned char* to) {        // any k0: the pages are kept inside the needed ones
+  // any k0: the pages are kept inside the needed ones
+  auto load_tile = [&](int k0, unsigned char* to) __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < LOADS; ++it) {
       load_k(k0 & (page_size - 1), it, to);
@@ -177,7 +185,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     held = look_up(k0 + BK);
   };
   // Values of keys outside [key_begin, key_end) of the tile at `tile` become zero (K needs none: the mask).
-  auto zero_values = [&](int k0, unsigned char* tile) {
+  auto zero_values = [&](int k0, unsigned char* tile) __attribute__((always_inline)) {
     for (int idx = threadIdx.x; idx < BK / 8 * D; idx += THREADS) {
       const int key = k0 + idx / D * 8;
       if (key >= key_begin && key + 8 <= key_end) continue;
@@ -195,10 +203,10 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   const float c = scale * 1.44269504088896f;               // p = exp2((s - m) c): the scale enters in the exponent
   const uint32_t k_read = l32 * (D * 2), k_piece = half ^ (l32 & 15);        // piece 2 ks + half of row l32 is at (2 ks) ^ k_piece
   const uint32_t v_read = (half * D + l32) * 16;
-  auto attend = [&](int k0, const unsigned char* tile, unsigned char* next, bool masked) {
+  auto attend = [&](int k0, const unsigned char* tile, unsigned char* next, bool masked) __attribute__((always_inline)) {
     const unsigned char* Ks = tile + k_read;
     const unsigned char* Vt = tile + BK * D * 2 + v_read;
-    auto k_fragment = [&](int kt, int ks) {
+    auto k_fragment = [&](int kt, int ks) __attribute__((always_inline)) {
       return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Ks + kt * 32 * D * 2 + (((2 * ks) ^ k_piece) << 4)));
     };
     constexpr int AHEAD = 2;                               // steps of 16 dims whose fragments are on their way
@@ -245,11 +253,14 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
-    const float m_new = fmaxf(row_m, mx);
+    // the reference of the exponents moves (to the maximum) only if the maximum is 2^8 beyond it, or there was none
+    const bool moves = (mx - row_m) * c > 8.f || (row_m == -INFINITY && mx != -INFINITY);
+    const float m_new = moves ? mx : row_m;
     const float base = (m_new == -INFINITY) ? 0.f : m_new;                                // exp(-inf - 0) = 0
     const float shift = -base * c;
-    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(fmaf(row_m, c, shift));
-    if (m_new != row_m) {                        // nothing to rescale while the maximum stands
+    float alpha = 1.f;
+    if (__builtin_amdgcn_ballot_w64(moves) != 0) {
+      alpha = moves ? __builtin_amdgcn_exp2f(fmaf(row_m, c, shift)) : 1.f;                // exp2(-inf) = 0 at the first keys
 #pragma unroll
       for (int t = 0; t < WTILES; ++t)
 #pragma unroll
@@ -276,7 +287,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     }
     row_l = row_l * alpha + psum;
     asm volatile("" : "+v"(row_l));                        // summed here, not after the products below
-    auto v_fragment = [&](int u, int t) {
+    auto v_fragment = [&](int u, int t) __attribute__((always_inline)) {
       return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Vt + u * (2 * D * 16) + t * (32 * 16)));
     };
     bf16x8 va[4][WTILES];
@@ -299,12 +310,12 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   held = look_up(first_tile);
   load_tile(first_tile, lds);
   int buffer = 0;
-  for (int k0 = first_tile; k0 < key_end; k0 += BK, buffer ^= 1) {
+  auto tile_step = [&](int k0, auto edge_tag) __attribute__((always_inline)) {
     unsigned char* tile = lds + buffer * PROMPT_TILE_BYTES;
     unsigned char* next = lds + (buffer ^ 1) * PROMPT_TILE_BYTES;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's loads of the tile have landed
     __syncthreads();                                       // everyone's have, and everyone is done with the tile before
-    if (!(k0 >= key_begin && k0 + BK <= key_end)) {
+    if (decltype(edge_tag)::value && !(k0 >= key_begin && k0 + BK <= key_end)) {
       zero_values(k0, tile);
       __syncthreads();
     }
@@ -315,7 +326,13 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     } else {
       load_tile(k0 + BK, next);
     }
-  }
+    buffer ^= 1;
+  };
+  // only the first and the last tile can hold keys outside [key_begin, key_end): the loop between has no such check
+  int k0 = first_tile;
+  tile_step(k0, std::true_type());
+  for (k0 += BK; k0 + BK < key_end; k0 += BK) tile_step(k0, std::false_type());
+  if (k0 < key_end) tile_step(k0, std::true_type());
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // no load into LDS is on its way when the block ends
 
   if (!wave_active) return;

@@ -538,12 +538,14 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
     return launch_fast<64, 2, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);
   // Head size 128 has a kernel of its own (attention_prompt.hip).  Blocks of 8 waves (64 rows of 4 heads, or 128 of
-  // 2, ... share a staged tile of keys; one block a CU) once blocks of 4 waves would be four or more a CU.
+  // 2, ... share a staged tile of keys; one block a CU) once blocks of 4 waves would be eight or more a CU: measured
+  // with 32 heads in 8 groups, 4 waves against 8: 58 : 68 us at 2,048 tokens, 172 : 191 at 4,096, 610 : 563 at
+  // 8,192, 2,144 : 2,004 at 16,384.
   if (d == 128) {
     const int g128 = heads / kv_heads, gh128 = g128 >= 3 ? 4 : g128;
     const long blocks4 = (long)((max_query + 32 * (4 / gh128) - 1) / (32 * (4 / gh128))) * n_seqs * kv_heads *
                          ((g128 + gh128 - 1) / gh128);
-    const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 1024;
+    const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 2048;
     return qil_attn_prompt(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
                            max_query, heads, kv_heads, page_size, window, scale, wide ? 8 : 4, nullptr, 0, 0, 1, s);
   }
