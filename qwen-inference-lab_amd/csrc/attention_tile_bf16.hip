@@ -1,7 +1,7 @@
-// The tile kernel of attention_tile.hip for its common case, written without branches in the tile loop:
-// bfloat16, head size exactly D (64, 128 or 256), a page size that is a power of two from 8 on, a block
-// table of a sequence that fits in LDS.  Same block shape, same matrix-core formulation, same order of every sum, so a row gets
-// bit for bit the result of the general kernel (qil/model.py:59-66 is the formula of both).
+// The tile kernel of attention_tile.hip for common cases, written without branches in the tile loop: bfloat16, head
+// size exactly D (64 or 256; 128 goes on to attention_prompt.hip from here), a page size that is a power of two from
+// 8 on, a block table of a sequence that fits in LDS.  Same block shape, same matrix-core formulation, same order of
+// every sum, so a row gets bit for bit the result of the general kernel (qil/model.py:59-66 is the formula of both).
 //
 // What differs is the schedule:
 //  * the sequence's block-table entries are copied to LDS once, so finding a page is an LDS read and

@@ -632,6 +632,43 @@ def test_prompt_portions_against_float64(ops, dtype, lengths, chunks, page_size,
     mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, None, scale=d ** -0.5)
 
 
+@pytest.mark.parametrize('growth', [0.02, 0.11, 1.5])
+@pytest.mark.parametrize('waves', [4, 8])
+def test_prompt_attention_with_scores_that_grow_along_the_keys(ops, growth, waves):
+    """The kernel for head size 128 keeps a row's reference exponent until a score exceeds it by 2^8.  Keys whose
+    scores grow by `growth` (in the exponent, to base 2) from one key to the next move it never within a tile's
+    reach, every few tiles, or at every tile: probabilities up to 2^8 and rescaled sums, against float64."""
+    page_size, d, heads, kv_heads, n, rows = 16, 128, 8, 2, 1200, 330
+    k_cache, v_cache, table, histories = build_cache([n], page_size, kv_heads, d, torch.bfloat16)
+    torch.manual_seed(5)
+    direction = torch.nn.functional.normalize(torch.randn(kv_heads, d), dim=-1)
+    j = torch.arange(n, dtype=torch.float32)
+    k = (0.05 * torch.randn(n, kv_heads, d) + j[:, None, None] * 0.01 * direction).to(torch.bfloat16)
+    page = table[0].cpu()[(j.long() // page_size)].long()
+    k_cache[page.cuda(), :, (j.long() % page_size).cuda()] = k.cuda()
+    histories[0] = (k, histories[0][1])
+    scale = 1.0
+    # a query along the direction: score of key j = j * 0.01 * |q|, so |q| = growth / (0.01 * log2(e))
+    g = heads // kv_heads
+    q = torch.stack([direction[h // g] * (growth / (0.01 * 1.4426950408889634)) for h in range(heads)])
+    qkv = (q[None] + 0.02 * torch.randn(rows, heads, d)).to(torch.bfloat16).reshape(rows, heads * d).cuda()
+    start = n - rows
+    dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
+    lib = ops.library.load()
+    lib.qil_attn_tile_waves(waves)
+    try:
+        got = ops.paged_attention(qkv, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                                  page_size=page_size, block_tables=table, row_seq=dev([0] * rows),
+                                  positions=dev(list(range(start, n))), cu_seqlens=dev([0, rows]), seq_starts=dev([start]),
+                                  single_rows=dev([]), n_seqs=1, max_query=rows, max_context=n, scale=scale, window=None)
+    finally:
+        lib.qil_attn_tile_waves(0)
+    expected = plain.attention(qkv.reshape(rows, heads, d).double().cpu(), k.double(), histories[0][1].double(),
+                               torch.arange(start, n), scale).reshape(rows, heads * d)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.double().cpu(), expected, **ATT_TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize('lengths,chunks,heads,kv_heads,window', [
     ([700, 90, 33], [700, 31, 33], 16, 4, None),                # g = 4: 64 rows of 4 heads a block
     ([513, 200], [300, 200], 8, 4, None),                       # g = 2: 128 rows of 2 heads
