@@ -1,0 +1,289 @@
+// bfloat16 products of 65 to 256 rows (a portion of a prompt beside decoded rows, a large decode batch, a short
+// prompt):  C[M, N] = A[M, K] W[N, K]^T, float32 accumulation.  Such a product reads its weights once, like the
+// few-row products, but has work for the matrix cores at a third to a half of their rate.
+//
+//  * A wave owns 32 columns of C and all rows: per 16 columns of K it reads one fragment of W and M / 32 fragments
+//    of A from LDS and makes M / 32 products v_mfma_f32_32x32x16_bf16 (a 16 x 16 x 32 product needs twice the LDS
+//    bytes for the same work).
+//  * W and A go from memory straight into LDS (global_load_lds_dwordx4, whole 128-byte lines, no registers): W into
+//    a ring of the wave's own, A into a ring that the block's multiplying waves share and a wave of its own fills
+//    (one barrier a stage of 64 columns of K).  Piece p of row r holds the columns 8 (p ^ (r & 7)) ..: fragment
+//    reads spread over the banks.
+//  * A block is 2 to 4 multiplying waves (64 to 128 columns) and K is split over blocks, so that the blocks fill
+//    whole rounds of the 256 CUs (a block holds a CU's LDS); float32 partial sums [split][M][N] are added by the
+//    kernel that consumes them, as those of the few-row products are.  With one split the result is written in the
+//    model's type, and for a gated feed-forward's first product (gate and up rows in turns of 16) as
+//    silu(gate) * up.
+// Takes N a multiple of 32, K a multiple of 64 with at least 4 stages a split, 16-byte aligned operands.
+// Measured at 160 rows and Qwen3-8B sizes (q/k/v, attention output, gate/up, down): 19, 15, 53, 30 us against 30,
+// 18, 55 + 5 (activation), 40 of the kernels it replaces there; a stage still takes 1,500 cycles where its 20
+// products take 640.
+#include <algorithm>
+
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define MID_STAGE 64                                       // columns of K a stage: rows of 128 bytes
+#define MID_WAVES 4
+#define MID_COLS (32 * MID_WAVES)                          // columns of C a block
+#define MID_MOST_ROWS 256
+#define MID_LDS_LIMIT (156 * 1024)
+
+// Stages in LDS.  W streams from memory at full rate with two stages (8 KB a wave) on their way; A comes from L2
+// and is what the barrier waits for, two stages after it was sent: a stage's time is then at least half of that
+// latency (under load 3,000 cycles and more), however little there is to multiply.  So W gets three or four places
+// and A as many as fit beside them, at most 8.
+__host__ __device__ constexpr int mid_w_ring(int mt) { return mt <= 6 ? 4 : 3; }
+__host__ __device__ constexpr int mid_a_ring(int mt) {
+  const int fit = (MID_LDS_LIMIT - mid_w_ring(mt) * MID_WAVES * 4096) / (mt * 4096);
+  return fit < 8 ? fit : 8;
+}
+
+// MT: row tiles of 32 (M <= 32 MT).  OUT: float (partial sums or the result) or bf16_t (the result, one split).
+// GATED (one split): W holds gate and up rows in turns of 16, a wave's 32 columns are 16 of each, and C [M, N / 2]
+// gets silu(gate) * up (qil/model.py:71), both still in float32.
+// Waves 0 to 3 multiply, each with a ring of W of its own; wave 4 loads A for all of them.  A wave waits for its
+// loads by their number in flight (vmcnt counts in order), so loads that must land soon (A, from L2, three stages
+// in LDS) and loads that are sent far ahead (W, from memory) belong to different waves.
+template <int MT, typename OUT, bool GATED>
+__global__ void __launch_bounds__((MID_WAVES + 1) * QIL_WAVE, 1)
+gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N, int K,
+                     int stages, int waves) {
+  constexpr int RW = mid_w_ring(MT), RA = mid_a_ring(MT);
+  constexpr int W_SLOT = MID_WAVES * 4096, A_SLOT = MT * 4096;   // bytes of a stage: 32 rows x 128 bytes a wave; 32 MT rows
+  extern __shared__ __align__(1024) unsigned char lds[];   // W ring, then A ring
+  unsigned char* a_ring = lds + RW * W_SLOT;
+  const int lane = threadIdx.x & (QIL_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / QIL_WAVE);
+  const size_t k_begin = (size_t)blockIdx.y * stages * MID_STAGE;
+  // loads: a load is 8 rows of 128 bytes; lane = (row lane / 8, place lane % 8), and place p of row r takes piece p ^ (r & 7)
+  const int rl = lane >> 3;
+  const uint32_t piece_bytes = ((lane & 7) ^ rl) << 4;
+
+  if (wave == waves) {                                     // ---- the wave that loads A (the last of the block)
+    const char* a_from = reinterpret_cast<const char*>(A + k_begin) + piece_bytes;
+    uint32_t a_row_bytes[4 * MT];                          // rows past the last read it again: their results are not stored
+#pragma unroll
+    for (int j = 0; j < 4 * MT; ++j) a_row_bytes[j] = (uint32_t)min(8 * j + rl, M - 1) * (uint32_t)K * 2;
+    auto load_a = [&](int stage) __attribute__((always_inline)) {
+      const size_t at = (size_t)stage * (MID_STAGE * 2);
+      unsigned char* a_to = a_ring + (stage % RA) * A_SLOT;
+#pragma unroll
+      for (int j = 0; j < 4 * MT; ++j)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_from + at + a_row_bytes[j]),
+                                         (__attribute__((address_space(3))) void*)(a_to + j * 1024), 16, 0, 0);
+    };
+#pragma unroll
+    for (int s = 0; s < RA - 1; ++s)
+      if (s < stages) load_a(s);
+    for (int stage = 0; stage < stages; ++stage) {
+      // all but the newest RA - 2 stages have landed (near the end: all); after the barrier everyone is done with
+      // the stage before, whose place the next loads take
+      if (stage + RA - 2 < stages) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((RA - 2) * 4 * MT) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      if (stage + RA - 1 < stages) load_a(stage + RA - 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+
+  // ---- the waves that multiply
+  const int l32 = lane & 31, half = lane >> 5;
+  const int n0 = (blockIdx.x * waves + wave) * 32;         // the wave's columns (a wave past the end repeats the last ones)
+  const int n_load = min(n0, N - 32);
+  const char* w_from = reinterpret_cast<const char*>(W + (size_t)(n_load + rl) * K + k_begin) + piece_bytes;
+  const size_t w_rows8 = (size_t)8 * K * 2;
+  auto load_w = [&](int stage) __attribute__((always_inline)) {
+    const size_t at = (size_t)stage * (MID_STAGE * 2);
+    unsigned char* w_to = lds + (stage % RW) * W_SLOT + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_from + at + i * w_rows8),
+                                       (__attribute__((address_space(3))) void*)(w_to + i * 1024), 16, 0, 0);
+  };
+  // fragment reads: lane = (row lane % 32, half lane / 32) wants piece 2 ks + half of its row: at place (2 ks) ^ (half ^ (row & 7))
+  const uint32_t piece = half ^ (l32 & 7);
+  uint32_t read_at[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) read_at[ks] = l32 * 128 + (((2 * ks) ^ piece) << 4);
+
+  f32x16 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+
+#pragma unroll
+  for (int s = 0; s < RW - 1; ++s)
+    if (s < stages) load_w(s);
+  for (int stage = 0; stage < stages; ++stage) {
+    // this wave's W of the stage has landed when all but the newest RW - 2 stages' loads have (near the end: all);
+    // after the barrier A has too
+    if (stage + RW - 2 < stages) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((RW - 2) * 4) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (stage + RW - 1 < stages) load_w(stage + RW - 1);
+    const unsigned char* w_at = lds + (stage % RW) * W_SLOT + wave * 4096;
+    const unsigned char* a_at = a_ring + (stage % RA) * A_SLOT;
+    // the fragments of the next 16 columns are read while these are multiplied (one wave a SIMD: nobody else hides
+    // the LDS latency)
+    bf16x8 wf[4], af[4][MT];
+    auto fragments = [&](int ks) __attribute__((always_inline)) {
+      wf[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(w_at + read_at[ks]));
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        af[ks][t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(a_at + t * 4096 + read_at[ks]));
+    };
+    fragments(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks + 1 < 4) fragments(ks + 1);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks], af[ks][t], acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // acc[t][e]: row m = 32 t + l32, column n0 + 8 (e / 4) + 4 half + e % 4
+  if (n0 >= N) return;
+  if constexpr (GATED) {                                   // columns 0-15 of the wave are gates, 16-31 the ups that belong to them
+    const int inner = N / 2;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = 32 * t + l32;
+      if (m >= M) continue;
+      OUT* row = C + (size_t)m * inner + n0 / 2 + 4 * half;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float gate = acc[t][4 * g + e];
+          v[e] = (gate / (1.f + expf(-gate))) * acc[t][4 * (g + 2) + e];
+        }
+        if constexpr (sizeof(OUT) == 4) *reinterpret_cast<float4*>(row + 8 * g) = make_float4(v[0], v[1], v[2], v[3]);
+        else *reinterpret_cast<uint2*>(row + 8 * g) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+      }
+    }
+    return;
+  }
+  OUT* out = C + (size_t)blockIdx.y * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = 32 * t + l32;
+    if (m >= M) continue;
+    OUT* row = out + (size_t)m * N + n0 + 4 * half;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if constexpr (sizeof(OUT) == 4)
+        *reinterpret_cast<float4*>(row + 8 * g) = make_float4(acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]);
+      else
+        *reinterpret_cast<uint2*>(row + 8 * g) =
+            make_uint2(pack_bf16(acc[t][4 * g], acc[t][4 * g + 1]), pack_bf16(acc[t][4 * g + 2], acc[t][4 * g + 3]));
+    }
+  }
+}
+
+// Multiplying waves a block (2 to 4: 64 to 128 columns) and splits of K for these sizes; false if the kernel does not
+// take them.  A block holds a CU (its LDS), so the blocks should fill whole rounds of the 256 CUs: of the plans with
+// whole stages, 4 stages or more a split and at most 16 splits, the one with the least time by this count (rounds
+// times a block's stages, a little for every split's partial sums) is taken; splits: 0 = free, else given.
+static bool mid_plan(int M, int N, int K, int* waves, int* splits) {
+  if (M < 1 || M > MID_MOST_ROWS || N < 32 || N % 32 || K < 4 * MID_STAGE || K % MID_STAGE) return false;
+  const int stages = K / MID_STAGE, given = *splits;
+  double best = 0;
+  bool found = false;
+  for (int w = MID_WAVES; w >= 2; --w)
+    for (int sp = 1; sp <= 16; ++sp) {
+      if ((given && sp != given) || stages % sp || stages / sp < 4) continue;
+      const long blocks = (long)((N / 32 + w - 1) / w) * sp;
+      const long rounds = (blocks + 255) / 256;
+      // a block's time: its stages, each as long as its W takes at the CU's share of the memory's rate, but not
+      // shorter than what a stage costs anyway (barrier, sending the loads, the first fragments); CUs without a block
+      // are memory streams that are missing
+      const double idle = blocks < 256 ? 0.3 * (256 - blocks) / 256.0 : 0.0;
+      const double cost = (double)rounds * (stages / sp + 6) * std::max(3.5, (double)w) * (1.0 + idle) + 0.02 * sp * stages;
+      if (!found || cost < best) { best = cost; *waves = w; *splits = sp; found = true; }
+    }
+  return found;
+}
+
+template <int MT, typename OUT, bool GATED>
+static int mid_launch(const void* A, const void* W, void* C, int M, int N, int K, int waves, int splits, hipStream_t s) {
+  const size_t lds = (size_t)mid_w_ring(MT) * MID_WAVES * 4096 + (size_t)mid_a_ring(MT) * MT * 4096;
+  auto kernel = gemm_bf16_mid_kernel<MT, OUT, GATED>;
+  static bool granted = false;                             // per instantiation
+  if (!granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = true;
+  }
+  dim3 grid((N / 32 + waves - 1) / waves, splits);
+  hipLaunchKernelGGL(kernel, grid, dim3((waves + 1) * QIL_WAVE), lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)C, M, N, K,
+                     K / MID_STAGE / splits, waves);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+template <bool GATED>
+static int mid_dispatch(const void* A, const void* W, void* C, int M, int N, int K, int out_dtype, int waves, int splits,
+                        hipStream_t s) {
+#define QIL_MID_CASE(MT)                                                                                      \
+  case MT:                                                                                                    \
+    return out_dtype == QIL_F32 ? mid_launch<MT, float, GATED>(A, W, C, M, N, K, waves, splits, s)            \
+                                : mid_launch<MT, bf16_t, GATED>(A, W, C, M, N, K, waves, splits, s)
+  switch ((M + 31) / 32) {
+    QIL_MID_CASE(1);
+    QIL_MID_CASE(2);
+    QIL_MID_CASE(3);
+    QIL_MID_CASE(4);
+    QIL_MID_CASE(5);
+    QIL_MID_CASE(6);
+    QIL_MID_CASE(7);
+    QIL_MID_CASE(8);
+  }
+#undef QIL_MID_CASE
+  return -1;
+}
+
+extern "C" {
+
+// Splits of K that qil_gemm_bf16_mid uses for these sizes; 0 if it does not take them.
+int qil_gemm_bf16_mid_splits(int M, int N, int K) {
+  int waves = 0, splits = 0;
+  return mid_plan(M, N, K, &waves, &splits) ? splits : 0;
+}
+
+// C = A[M, K] W[N, K]^T for 1 <= M <= 256.  splits > 1: C float32 [splits][M][N] partial sums (out_dtype QIL_F32);
+// splits == 1: C [M][N] of out_dtype.  splits: 0 = chosen here (qil_gemm_bf16_mid_splits), else a divisor of K / 64
+// that leaves 4 stages or more.
+int qil_gemm_bf16_mid(const void* A, const void* W, void* C, int M, int N, int K, int out_dtype, int splits, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  int waves = 0;
+  if (splits < 0 || splits > 16 || !mid_plan(M, N, K, &waves, &splits) || ((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) % 16)
+    return -1;
+  if ((splits > 1 && out_dtype != QIL_F32) || (out_dtype != QIL_F32 && out_dtype != QIL_BF16)) return -1;
+  return mid_dispatch<false>(A, W, C, M, N, K, out_dtype, waves, splits, s);
+}
+
+// 1 if qil_gemm_bf16_mid_gated takes these sizes: those of the product with 2 * inner columns, which in one split must
+// give every CU work.
+int qil_gemm_bf16_mid_gated_takes(int M, int inner, int K) {
+  int waves = 0, splits = 1;
+  return inner >= 16 && inner % 16 == 0 && mid_plan(M, 2 * inner, K, &waves, &splits) &&
+         (2 * inner / 32 + waves - 1) / waves >= 192;
+}
+
+// out [M, inner] of out_dtype = silu(A gate^T) * (A up^T) for W [2 inner, K] with gate and up rows in turns of 16.
+int qil_gemm_bf16_mid_gated(const void* A, const void* W, void* out, int M, int inner, int K, int out_dtype, hipStream_t s) {
+  if (M == 0 || inner == 0) return 0;
+  int waves = 0, splits = 1;
+  if (!qil_gemm_bf16_mid_gated_takes(M, inner, K) || !mid_plan(M, 2 * inner, K, &waves, &splits) ||
+      ((uintptr_t)A | (uintptr_t)W | (uintptr_t)out) % 16 || (out_dtype != QIL_F32 && out_dtype != QIL_BF16))
+    return -1;
+  return mid_dispatch<true>(A, W, out, M, 2 * inner, K, out_dtype, waves, 1, s);
+}
+
+}  // extern "C"

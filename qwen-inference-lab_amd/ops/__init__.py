@@ -24,6 +24,7 @@ STREAM_GEMM_MAX_ROWS = 16
 # (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
 # the library says which products it takes (those of few column tiles), and of 129 to 192 rows.
 STREAM_GEMM_MOST_ROWS = 192
+MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 65, 256   # products of the 32 x 32 kernel with operands loaded straight into LDS
 # Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
 ATTENTION_PART = 256
 # Blocks the row attention kernel aims for.
@@ -291,6 +292,13 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False, add_to=None):
         _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, splits, _stream()), 'gemm_f32')
         return Partials(out) if splits > 1 else out[0]
     _code(x.dtype)
+    if MID_GEMM_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS and bias is None and out_dtype == x.dtype:
+        splits = lib.qil_gemm_bf16_mid_splits(n, o, k)
+        if splits == 1 or (splits > 1 and partials):
+            out = torch.empty((splits, n, o), dtype=torch.float32 if splits > 1 else x.dtype, device=x.device)
+            _check(lib.qil_gemm_bf16_mid(_ptr(x), _ptr(weight), _ptr(out), n, o, k, _code(out.dtype), splits, _stream()),
+                   'gemm_bf16_mid')
+            return Partials(out) if splits > 1 else out[0]
     streams = n <= STREAM_GEMM_MOST_ROWS and bool(lib.qil_gemm_bf16_streams(n, o, k, bias is not None))
     if streams and partials and bias is None and out_dtype == x.dtype:
         splits = lib.qil_gemm_bf16_splits(n, o, k)
@@ -323,7 +331,7 @@ def gated_linear(x, weight, out_dtype=None, interleaved=False):
     """silu(x @ gate^T) * (x @ up^T) -> [N, I], with ``weight`` the [2 I, K] matrix of both: the gate rows stacked
     before the up rows, or (``interleaved``) both in turns of 16 rows, which the kernels read faster.
 
-    One kernel when a fused kernel takes the sizes (bfloat16; up to 16 rows, or up to 64 rows of an interleaved
+    One kernel when a fused kernel takes the sizes (bfloat16; up to 16 rows, or up to 256 rows of an interleaved
     matrix large enough to fill the chip); otherwise the product followed by ``silu_mul``.  Both add in float32."""
     if isinstance(x, Normed):
         x = x.materialize()
@@ -339,6 +347,12 @@ def gated_linear(x, weight, out_dtype=None, interleaved=False):
         out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
         _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
                                        int(interleaved), _stream()), 'gemm_bf16_gated')
+        return out
+    if x.dtype == torch.bfloat16 and interleaved and MID_GEMM_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS and \
+            lib.qil_gemm_bf16_mid_gated_takes(n, both // 2, k):
+        out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
+        _check(lib.qil_gemm_bf16_mid_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), _stream()),
+               'gemm_bf16_mid_gated')
         return out
     return silu_mul(linear(x, weight, None, partials=True), out_dtype, interleaved=interleaved)
 

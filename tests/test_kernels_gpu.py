@@ -309,6 +309,80 @@ def test_gated_linear(ops, m, inner, k, dtype):
         check(ops.silu_mul(y_turns, interleaved=True), ops.silu_mul((x.double() @ w.double().t()).to(dtype)), dtype, scale=0)
 
 
+@pytest.mark.parametrize('m', [1, 31, 33, 65, 96, 128, 129, 160, 161, 200, 256])
+@pytest.mark.parametrize('n,k', [(4096, 4096), (6144, 1024), (96, 256), (160, 4160), (24576, 512), (32, 320)])
+def test_products_of_up_to_256_rows_loaded_straight_into_lds(ops, m, n, k):
+    """The kernel for 65 to 256 rows (it takes fewer too): 32 x 32 x 16 products, W and A loaded straight into LDS, a
+    wave of its own for A, K split over blocks.  Every plan it makes (2 to 4 multiplying waves, 1 to 16 splits)
+    and forced splits, partial sums and direct results in both types, against float64; and through the op."""
+    lib = ops.library.load()
+    x = rand(m, k, dtype=torch.bfloat16)
+    w = rand(n, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
+    want = x.double() @ w.double().t()
+    raw = torch.cuda.current_stream().cuda_stream
+    planned = lib.qil_gemm_bf16_mid_splits(m, n, k)
+    assert 1 <= planned <= 16 and (k // 64) % planned == 0 and k // 64 // planned >= 4
+    for splits in sorted({planned, 1, 2, 5, 16}):
+        stages = k // 64
+        takes = stages % splits == 0 and stages // splits >= 4
+        out = torch.full((splits, m, n), float('nan'), dtype=torch.float32, device='cuda')
+        status = lib.qil_gemm_bf16_mid(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k, 0, splits, raw)
+        assert status == (0 if takes else -1), (splits, status)
+        if takes:
+            assert torch.isfinite(out).all()
+            torch.testing.assert_close(out.double().sum(0).cpu(), want.cpu(), atol=3e-6 * want.abs().max().item(), rtol=1e-4)
+    direct = torch.full((m, n), float('nan'), dtype=torch.bfloat16, device='cuda')
+    assert lib.qil_gemm_bf16_mid(x.data_ptr(), w.data_ptr(), direct.data_ptr(), m, n, k, 1, 1, raw) == 0
+    check(direct, want, torch.bfloat16, scale=8)
+    assert lib.qil_gemm_bf16_mid(x.data_ptr(), w.data_ptr(), direct.data_ptr(), m, n, k, 1, 2, raw) == -1   # partial sums are float32
+    got = ops.linear(x, w, None, partials=True)
+    if isinstance(got, ops.Partials):
+        torch.testing.assert_close(got.sum().double().cpu(), want.cpu(), atol=3e-6 * want.abs().max().item(), rtol=1e-4)
+    else:
+        check(got, want, torch.bfloat16, scale=8)
+    check(ops.linear(x, w), want, torch.bfloat16, scale=8)
+
+
+def test_products_of_up_to_256_rows_refuse_other_sizes(ops):
+    lib = ops.library.load()
+    assert lib.qil_gemm_bf16_mid_splits(257, 4096, 4096) == 0                    # rows
+    assert lib.qil_gemm_bf16_mid_splits(128, 4100, 4096) == 0                    # columns in whole waves
+    assert lib.qil_gemm_bf16_mid_splits(128, 4096, 4000) == 0                    # K in whole stages
+    assert lib.qil_gemm_bf16_mid_splits(128, 4096, 192) == 0                     # four stages at least
+    x = rand(128, 192, dtype=torch.bfloat16)
+    w = rand(64, 192, dtype=torch.bfloat16, seed=1)
+    check(ops.linear(x, w), x.double() @ w.double().t(), torch.bfloat16, scale=8)   # the op finds another way
+
+
+@pytest.mark.parametrize('m', [65, 100, 160, 256])
+@pytest.mark.parametrize('inner,k', [(12288, 4096), (6144, 256), (9216, 320)])
+def test_gated_linear_of_65_to_256_rows(ops, m, inner, k):
+    """The same kernel with the gate's epilogue: a wave's 32 columns are 16 gates and their 16 ups (rows in turns of
+    16), one split, the result written once.  Against float64 and against the product followed by the activation."""
+    lib = ops.library.load()
+    x = rand(m, k, dtype=torch.bfloat16)
+    stacked = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
+    y = x.double() @ stacked.double().t()
+    want = torch.nn.functional.silu(y[:, :inner]) * y[:, inner:]
+    w = ops.interleave_gate_up(stacked[:inner].contiguous(), stacked[inner:].contiguous())
+    assert lib.qil_gemm_bf16_mid_gated_takes(m, inner, k)
+    assert not lib.qil_gemm_bf16_mid_gated_takes(m, 1024, k)                     # too few columns for one split
+    raw = torch.cuda.current_stream().cuda_stream
+    for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
+        out = torch.full((m, inner), float('nan'), dtype=dtype, device='cuda')
+        assert lib.qil_gemm_bf16_mid_gated(x.data_ptr(), w.data_ptr(), out.data_ptr(), m, inner, k, code, raw) == 0
+        if dtype == torch.float32:
+            assert torch.isfinite(out).all()
+            torch.testing.assert_close(out.double().cpu(), want.cpu(), atol=2e-6 * want.abs().max().item(), rtol=1e-4)
+        else:
+            check(out, want, dtype, scale=8)
+    got = ops.gated_linear(x, w, interleaved=True)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, inner)
+    check(got, want, torch.bfloat16, scale=8)
+    unfused = ops.silu_mul(ops.linear(x, w, None, partials=True), torch.bfloat16, interleaved=True)
+    check(unfused, want, torch.bfloat16, scale=8)
+
+
 @pytest.mark.parametrize('m', [17, 32, 33, 64, 65, 96, 100, 128, 129, 160, 161, 192])
 @pytest.mark.parametrize('inner,k', [(12288, 4096), (8192, 1024), (8208, 384), (80, 512)])
 def test_gated_linear_of_17_to_192_rows(ops, m, inner, k):
