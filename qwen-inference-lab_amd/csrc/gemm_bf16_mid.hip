@@ -1,4 +1,4 @@
-// bfloat16 products of 65 to 256 rows (a portion of a prompt beside decoded rows, a large decode batch, a short
+// bfloat16 products of 33 to 256 rows (a portion of a prompt beside decoded rows, a large decode batch, a short
 // prompt):  C[M, N] = A[M, K] W[N, K]^T, float32 accumulation.  Such a product reads its weights once, like the
 // few-row products, but has work for the matrix cores at a third to a half of their rate.
 //

@@ -24,7 +24,7 @@ STREAM_GEMM_MAX_ROWS = 16
 # (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
 # the library says which products it takes (those of few column tiles), and of 129 to 192 rows.
 STREAM_GEMM_MOST_ROWS = 192
-MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 65, 256   # products of the 32 x 32 kernel with operands loaded straight into LDS
+MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 33, 256   # products of the 32 x 32 kernel with operands loaded straight into LDS
 # Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
 ATTENTION_PART = 256
 # Blocks the row attention kernel aims for.
