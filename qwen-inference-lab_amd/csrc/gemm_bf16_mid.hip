@@ -30,6 +30,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define MID_COLS (32 * MID_WAVES)                          // columns of C a block
 #define MID_MOST_ROWS 256
 #define MID_LDS_LIMIT (156 * 1024)
+// Starting stages of the blocks of a product whose K is not split (split parts read different bands already).
+// Measured at Qwen3-8B's gate/up sizes, 40 / 96 / 160 rows: 44 / 46 / 54 us with 1, 38 / 41 / 51 with 4 and with 16;
+// with 64 the blocks of an XCD want all of A at once and larger products lose.
+#define MID_TURNS 4
 
 // Stages in LDS.  W streams from memory at full rate with two stages (8 KB a wave) on their way; A comes from L2
 // and is what the barrier waits for, two stages after it was sent: a stage's time is then at least half of that
@@ -50,7 +54,7 @@ __host__ __device__ constexpr int mid_a_ring(int mt) {
 template <int MT, typename OUT, bool GATED>
 __global__ void __launch_bounds__((MID_WAVES + 1) * QIL_WAVE, 1)
 gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N, int K,
-                     int stages, int waves) {
+                     int stages, int waves, int turns) {
   constexpr int RW = mid_w_ring(MT), RA = mid_a_ring(MT);
   constexpr int W_SLOT = MID_WAVES * 4096, A_SLOT = MT * 4096;   // bytes of a stage: 32 rows x 128 bytes a wave; 32 MT rows
   extern __shared__ __align__(1024) unsigned char lds[];   // W ring, then A ring
@@ -58,6 +62,10 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
   const int lane = threadIdx.x & (QIL_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / QIL_WAVE);
   const size_t k_begin = (size_t)blockIdx.y * stages * MID_STAGE;
+  // With `turns` > 1 the blocks begin at that many different stages of K and wrap round (blocks of one XCD, every
+  // eighth, at the same one, so that its L2 holds one band of A): they then read different columns of K and not all
+  // the same narrow band of every row of W, which memory serves more slowly.
+  const int turned = (int)((blockIdx.x % (unsigned)turns) * stages / turns);
   // loads: a load is 8 rows of 128 bytes; lane = (row lane / 8, place lane % 8), and place p of row r takes piece p ^ (r & 7)
   const int rl = lane >> 3;
   const uint32_t piece_bytes = ((lane & 7) ^ rl) << 4;
@@ -68,7 +76,8 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
 #pragma unroll
     for (int j = 0; j < 4 * MT; ++j) a_row_bytes[j] = (uint32_t)min(8 * j + rl, M - 1) * (uint32_t)K * 2;
     auto load_a = [&](int stage) __attribute__((always_inline)) {
-      const size_t at = (size_t)stage * (MID_STAGE * 2);
+      const int k_stage = stage + turned < stages ? stage + turned : stage + turned - stages;
+      const size_t at = (size_t)k_stage * (MID_STAGE * 2);
       unsigned char* a_to = a_ring + (stage % RA) * A_SLOT;
 #pragma unroll
       for (int j = 0; j < 4 * MT; ++j)
@@ -96,7 +105,8 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
   const char* w_from = reinterpret_cast<const char*>(W + (size_t)(n_load + rl) * K + k_begin) + piece_bytes;
   const size_t w_rows8 = (size_t)8 * K * 2;
   auto load_w = [&](int stage) __attribute__((always_inline)) {
-    const size_t at = (size_t)stage * (MID_STAGE * 2);
+    const int k_stage = stage + turned < stages ? stage + turned : stage + turned - stages;
+    const size_t at = (size_t)k_stage * (MID_STAGE * 2);
     unsigned char* w_to = lds + (stage % RW) * W_SLOT + wave * 4096;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -223,7 +233,7 @@ static int mid_launch(const void* A, const void* W, void* C, int M, int N, int K
   }
   dim3 grid((N / 32 + waves - 1) / waves, splits);
   hipLaunchKernelGGL(kernel, grid, dim3((waves + 1) * QIL_WAVE), lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)C, M, N, K,
-                     K / MID_STAGE / splits, waves);
+                     K / MID_STAGE / splits, waves, splits == 1 ? MID_TURNS : 1);
   QIL_RETURN_LAUNCH_STATUS();
 }
 
