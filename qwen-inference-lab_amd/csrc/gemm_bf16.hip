@@ -266,7 +266,8 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, NormedA
     source[u] = W + (size_t)min(n0 + row, N - 1) * K + k_begin + piece * 8;
     place[u] = row * 128 + ((piece ^ row) & 15) * 8;
   }
-  // A slice first: its wait would otherwise cover the first stages of W as well
+  // A slice first: a wait for it after W's requests would cover the first stages of W as well (unless A goes
+  // straight into LDS, below)
   if (ASRC == 2) {
     // 1 / rms of the rows: wave m (and m + 8) adds the row's pieces lane by lane, then across the wave
     float* rstd = reinterpret_cast<float*>(lds + a_rows * row_width + LINES_WAVES * (16 * 128));
@@ -291,12 +292,24 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, NormedA
       }
       *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
     }
-  } else {
+  } else if (MERGE) {
     for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 8); idx += LINES_WAVES * QIL_WAVE) {
       const int m = idx / (cols_per_split / 8), c = (idx - m * (cols_per_split / 8)) * 8;
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (m < M) v = MERGE ? merged8(unmerged, m, k_begin + c) : *reinterpret_cast<const uint4*>(A + (size_t)m * K + k_begin + c);
+      if (m < M) v = merged8(unmerged, m, k_begin + c);
       *reinterpret_cast<uint4*>(a_lds + m * row_width + c) = v;
+    }
+  } else {
+    // A as it is goes from memory straight into LDS, 512 columns of a row an instruction, and is not waited for
+    // here: W's first stages are asked for right behind it (loads complete in order, so waiting for A later
+    // does not wait for them).  Rows past M repeat the last one; their products are never stored.
+    const int row_loads = (cols_per_split + 511) / 512;
+    for (int j = wave; j < a_rows * row_loads; j += LINES_WAVES) {
+      const int m = __builtin_amdgcn_readfirstlane(j / row_loads), c0 = __builtin_amdgcn_readfirstlane(j - m * row_loads) * 512;
+      if (c0 + lane * 8 < cols_per_split)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(A + (size_t)min(m, M - 1) * K + k_begin + c0 + lane * 8),
+            (__attribute__((address_space(3))) void*)(a_lds + m * row_width + c0), 16, 0, 0);
     }
   }
   // Every wave walks its K range from a start of its own and wraps around: waves that all read the
@@ -313,7 +326,15 @@ gemm_bf16_lines_kernel(const bf16_t* __restrict__ A, UnmergedA unmerged, NormedA
   request(w0, 0);                                           // the host sees to stages >= 3
   request(w1, 1);
   request(w2, 2);
-  __syncthreads();
+  if (ASRC == 0) {
+    // A has landed, W's 12 loads need not: s_waitcnt vmcnt(12) lgkmcnt(0).  As a builtin and with the LDS counter
+    // in it, because the compiler treats a load into LDS as an access of both kinds and, until it sees one wait
+    // that covers both counters, makes every later wait for a load a wait for all of them.
+    __builtin_amdgcn_s_waitcnt(0x07C);
+    __builtin_amdgcn_s_barrier();
+  } else {
+    __syncthreads();
+  }
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   // lanes past the kept rows read the rows again: their products are rows of D that are never stored
@@ -850,19 +871,23 @@ static void plan(int M, int N, int K, bool may_split, int* code, int* splits) {
     while (sp > 1 && steps / sp < 8) --sp;
     if (sp < 1) sp = 1;
     // up to 16 rows: of the splits the whole-line kernel takes (whole stages of 128 columns, at least LINES_DEPTH
-    // of them; up to 32), the one whose blocks fill their rounds of 256 CUs best, less 1.5 % a split for what the
-    // consumer of the partial sums reads.  One round of 160 blocks or more counts as full: measured, 160, 192,
-    // 256, 400 and 1,000 blocks stream equally well, 128, 280 and 320 (a last round a quarter full or less) 10 to
-    // 15 % slower, and 80 blocks 50 % slower than 380.
+    // of them; up to 32), the one with the least time by this count.  The blocks run in rounds of 256, one a CU; a
+    // block's stage takes a unit of time while at most 160 blocks share the memory and more in proportion beyond
+    // (measured: 160, 192, 256, 400 and 1,000 blocks stream equally well, 80 blocks take 50 % longer than 380); a
+    // block's start (its slice of A, the first stages on their way) costs two units (the 1,187 column blocks of
+    // Qwen3's logits: 226 us unsplit, 262 in four splits of 8 stages); every split adds 1.5 % for what the consumer
+    // of the partial sums reads.
     if (M <= 16 && K % 128 == 0) {
       int fit = 0;
-      double fit_score = 0;
+      double fit_time = 0;
       for (int c = 1; c <= 32; ++c) {
         if (K % (128 * c) || K / (128 * c) < LINES_DEPTH || lines_lds(M, K, c) > LINES_LDS_LIMIT) continue;
-        const long blocks = (long)column_blocks * c;
-        const long slots = blocks >= 160 && blocks <= 256 ? blocks : (blocks + 255) / 256 * 256;
-        const double score = (double)blocks / (double)slots - 0.015 * c;
-        if (!fit || score > fit_score) { fit = c; fit_score = score; }
+        const long blocks = (long)column_blocks * c, last = blocks % 256;
+        const int stages = K / (128 * c);
+        double time = (double)(blocks / 256) * (stages * 1.6 + 2.0);
+        if (last) time += stages * std::max(1.0, last / 160.0) + 2.0;
+        time *= 1.0 + 0.015 * c;
+        if (!fit || time < fit_time) { fit = c; fit_time = time; }
       }
       if (fit) sp = fit;
     }
