@@ -24,7 +24,10 @@ STREAM_GEMM_MAX_ROWS = 16
 # (gate/up), 24 against 37 (down), 15 against 17 (q/k/v), 11 against 15 (attention output).  Of 65 to 128 rows
 # the library says which products it takes (those of few column tiles), and of 129 to 192 rows.
 STREAM_GEMM_MOST_ROWS = 192
-MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 33, 256   # products of the 32 x 32 kernel with operands loaded straight into LDS
+# Rows of the products that go to the 32 x 32 kernel with operands loaded straight into LDS; with the gate's epilogue
+# it is ahead from 17 rows on, without it level with the staged kernel up to 32 rows.
+MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 33, 256
+MID_GATED_FEWEST_ROWS = 17
 # Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
 ATTENTION_PART = 256
 # Blocks the row attention kernel aims for.
@@ -343,16 +346,19 @@ def gated_linear(x, weight, out_dtype=None, interleaved=False):
         raise ValueError(f'gated_linear: x {tuple(x.shape)}, weight {tuple(weight.shape)}')
     out_dtype = out_dtype or x.dtype
     lib = library.load()
-    if x.dtype == torch.bfloat16 and n and lib.qil_gemm_bf16_gated_takes(n, both // 2, k, int(interleaved)):
-        out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
-        _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
-                                       int(interleaved), _stream()), 'gemm_bf16_gated')
-        return out
-    if x.dtype == torch.bfloat16 and interleaved and MID_GEMM_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS and \
+    # 17 to 256 rows of an interleaved matrix: the 32 x 32 tile kernel where it takes the sizes (measured against the
+    # staged 16 x 16 kernel with the same epilogue at 17 to 64 rows: 37 to 38 us against 38 to 43 at Qwen3-8B sizes,
+    # 73 to 85 against 87 to 102 at 14B sizes)
+    if x.dtype == torch.bfloat16 and interleaved and MID_GATED_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS and \
             lib.qil_gemm_bf16_mid_gated_takes(n, both // 2, k):
         out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
         _check(lib.qil_gemm_bf16_mid_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), _stream()),
                'gemm_bf16_mid_gated')
+        return out
+    if x.dtype == torch.bfloat16 and n and lib.qil_gemm_bf16_gated_takes(n, both // 2, k, int(interleaved)):
+        out = torch.empty((n, both // 2), dtype=out_dtype, device=x.device)
+        _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
+                                       int(interleaved), _stream()), 'gemm_bf16_gated')
         return out
     return silu_mul(linear(x, weight, None, partials=True), out_dtype, interleaved=interleaved)
 

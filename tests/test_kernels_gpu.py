@@ -354,11 +354,12 @@ def test_products_of_up_to_256_rows_refuse_other_sizes(ops):
     check(ops.linear(x, w), x.double() @ w.double().t(), torch.bfloat16, scale=8)   # the op finds another way
 
 
-@pytest.mark.parametrize('m', [65, 100, 160, 256])
+@pytest.mark.parametrize('m', [17, 32, 33, 64, 65, 100, 160, 256])
 @pytest.mark.parametrize('inner,k', [(12288, 4096), (6144, 256), (9216, 320)])
-def test_gated_linear_of_65_to_256_rows(ops, m, inner, k):
+def test_gated_linear_of_17_to_256_rows_on_32_x_32_tiles(ops, m, inner, k):
     """The same kernel with the gate's epilogue: a wave's 32 columns are 16 gates and their 16 ups (rows in turns of
-    16), one split, the result written once.  Against float64 and against the product followed by the activation."""
+    16), one split, the result written once; the op uses it from 17 rows on.  Against float64 and against the
+    product followed by the activation."""
     lib = ops.library.load()
     x = rand(m, k, dtype=torch.bfloat16)
     stacked = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
@@ -387,9 +388,9 @@ def test_gated_linear_of_65_to_256_rows(ops, m, inner, k):
 @pytest.mark.parametrize('inner,k', [(12288, 4096), (8192, 1024), (8208, 384), (80, 512)])
 def test_gated_linear_of_17_to_192_rows(ops, m, inner, k):
     """The gate's epilogue in the kernel that passes A through LDS in stages: a block owns 64 result columns, four
-    waves make the gate products and four the up products.  Where the op takes the sizes by itself (enough blocks to
-    fill the chip) it is that kernel that runs; small results are forced through it here.  Against float64, and
-    against the product followed by the activation."""
+    waves make the gate products and four the up products.  The op prefers the 32 x 32 tile kernel where that takes
+    the sizes, so this one is called directly, small results forced through it.  Against float64, and against the
+    product followed by the activation."""
     lib = ops.library.load()
     x = rand(m, k, dtype=torch.bfloat16)
     stacked = rand(2 * inner, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
