@@ -17,8 +17,9 @@ class StepEntry:
 class StepContext:
     """What parts see of a step.  Device tensors are int32.
 
-    Rows are the step's tokens, packed request after request in entry order;
-    ``cu_seqlens[s] .. cu_seqlens[s + 1]`` are the rows of sequence s.
+    Rows are the step's tokens, packed request after request in the order of ``requests``: the step function puts
+    the requests that bring several tokens first (``tile_seqs`` of them) and keeps the caller's order otherwise;
+    ``cu_seqlens[s] .. cu_seqlens[s + 1]`` are the rows of sequence s.  ``logit_rows`` follow the caller's order.
     """
     n_tokens: int
     n_seqs: int
@@ -37,6 +38,7 @@ class StepContext:
     host_starts: list = field(default_factory=list)
     host_slots: list = field(default_factory=list)
     requests: list = field(default_factory=list)
+    tile_seqs: int = None          # sequences 0 .. tile_seqs - 1 are those of two or more rows; None: any may be
 
 
 class StepPieces:

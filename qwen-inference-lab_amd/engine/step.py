@@ -69,6 +69,11 @@ class ModelRunner:
                    for e in entries]
         if validate:
             self._validate(entries)
+        # Requests that bring several tokens come first (the caller's order among them and among the others): the
+        # kernel for sequences of several rows then gets blocks for those sequences only.  The wanted places keep
+        # the caller's order.
+        given = entries
+        entries = sorted(given, key=lambda e: len(e.tokens) < 2)
         cache, ps = self.cache, self.cache.page_size
         starts = [cache.computed[e.request] for e in entries]
         for entry, start in zip(entries, starts):
@@ -81,7 +86,8 @@ class ModelRunner:
         tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=n)
         row_seq = np.repeat(np.arange(s), counts)
         positions = np.arange(n) - cu[row_seq] + np.asarray(starts)[row_seq]
-        logit_rows = np.fromiter((cu[i] + w for i, e in enumerate(entries) for w in e.want), dtype=np.int64)
+        first_row = {e.request: cu[i] for i, e in enumerate(entries)}
+        logit_rows = np.fromiter((first_row[e.request] + w for e in given for w in e.want), dtype=np.int64)
         slots = [cache.slots[e.request] for e in entries]
         single = cu[:-1][np.asarray(counts) == 1] if max(counts) > 1 else np.zeros(0, dtype=np.int64)
         pieces = StepPieces()
@@ -103,7 +109,8 @@ class ModelRunner:
             pieces.add(f'tables{index}', table.reshape(-1))
             pieces.add(f'token_slots{index}', token_slots)
         facts = dict(n=n, s=s, starts=starts, counts=counts, slots=slots, cu=cu.tolist(), widths=widths,
-                     max_context=int(max(st + c for st, c in zip(starts, counts))), n_logit_rows=len(logit_rows))
+                     max_context=int(max(st + c for st, c in zip(starts, counts))), n_logit_rows=len(logit_rows),
+                     tile_seqs=sum(c > 1 for c in counts))
         return entries, pieces, facts
 
     def _context(self, entries, pieces, facts, device_flat, max_context=None):
@@ -117,7 +124,7 @@ class ModelRunner:
             seq_slots=part('slots'), logit_rows=part('logit_rows'),
             single_rows=part('single_rows') if max(counts) > 1 else None, max_query=max(counts),
             max_context=max_context or facts['max_context'], host_cu_seqlens=facts['cu'], host_starts=facts['starts'],
-            host_slots=facts['slots'], requests=[e.request for e in entries])
+            host_slots=facts['slots'], requests=[e.request for e in entries], tile_seqs=facts['tile_seqs'])
         for view in self.views:
             if view is not None and hasattr(view, 'block_tables'):
                 view.block_tables = part(f'tables{view.group}').view(s, facts['widths'][view.group])

@@ -504,7 +504,7 @@ def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, pag
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False):
+                    unmerged=False, tile_seqs=None):
     """Attention of every row of the step over its request's cached keys.
 
     ``q`` [N, heads * head_dim] (head h at columns [h d, (h + 1) d)).  Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
@@ -514,6 +514,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
     kernel; rows alone in their sequence (``single_rows``: their indices, or None when every row is
     alone, i.e. ``max_query == 1``) go to the split-context row kernel.  With ``unmerged`` the result may
     come back as ``Unmerged`` (every row alone, context in several parts) for ``linear`` to merge.
+    ``tile_seqs``: the caller has put the sequences of two or more rows first and there are this many; the tile
+    kernel then gets blocks for these only (None: for every sequence; those of one row leave at once).
     """
     n = q.shape[0]
     qkv = q
@@ -536,19 +538,26 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             raise ValueError('single_rows must list the rows that are alone when some sequence has several')
         _require(single_rows, 'single_rows', torch.int32)
         # sequences of one row leave their blocks at once: only the others count for how full the chip is
-        part, parts = tile_key_parts(lib, qkv.dtype, max(1, n_seqs - single_rows.shape[0]), max_query, heads, kv_heads,
+        several = max(1, n_seqs - single_rows.shape[0])
+        if tile_seqs is not None:
+            if tile_seqs != n_seqs - single_rows.shape[0]:
+                raise ValueError('tile_seqs must count the sequences of two or more rows')
+            n_seqs = tile_seqs
+        part, parts = tile_key_parts(lib, qkv.dtype, several, max_query, heads, kv_heads,
                                      head_dim, page_size, block_tables.shape[1], max_context)
         if parts > 1:
             # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
             # rows of the step: what the merge leaves in rows that are alone is overwritten below)
-            workspace = torch.empty(lib.qil_attn_rows_workspace(n, heads, head_dim, parts) // 4, dtype=torch.float32,
+            # (with the sequences of several rows first, their rows are the step's first and the only ones merged)
+            merged = n if tile_seqs is None else n - single_rows.shape[0]
+            workspace = torch.empty(lib.qil_attn_rows_workspace(merged, heads, head_dim, parts) // 4, dtype=torch.float32,
                                     device=qkv.device)
             _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                 _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
-                                                _ptr(seq_starts), _ptr(workspace), n, n_seqs, max_query, heads,
+                                                _ptr(seq_starts), _ptr(workspace), merged, n_seqs, max_query, heads,
                                                 kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
                                                 parts, _stream()), 'attn_tile_parts')
-            _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), n, heads, head_dim,
+            _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), merged, heads, head_dim,
                                       int(window or 0), part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:
             _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),

@@ -75,6 +75,6 @@ class Attention(Mixer):
             q, k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
-            max_query=ctx.max_query, max_context=ctx.max_context,
+            max_query=ctx.max_query, max_context=ctx.max_context, tile_seqs=ctx.tile_seqs,
             scale=self.scale, window=self.window, unmerged=True, **sizes)
         return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

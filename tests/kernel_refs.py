@@ -94,7 +94,7 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False, accumulate=torch.float32):
+                    unmerged=False, tile_seqs=None, accumulate=torch.float32):
     n, d, g = q.shape[0], head_dim, heads // kv_heads
     qkv = q
     q = q.reshape(n, heads, d).to(accumulate)

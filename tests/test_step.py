@@ -152,6 +152,33 @@ def test_selected_rows_and_nothing_wanted(case):
     case.close(logits, expected[[8, 4]])
 
 
+def test_requests_with_several_tokens_come_first_and_logits_keep_the_callers_order(case):
+    """A step of single tokens and portions in turns: inside, the sequences of several rows are put first (the tile
+    kernel gets blocks for them alone), the logits come back in the order of the caller's entries and wants."""
+    config, weights, model, page_size = case
+    runner = ModelRunner(model, num_pages=64, page_size=page_size)
+    poison(runner)
+    lengths = {'a': 7, 'b': 12, 'c': 5, 'd': 9, 'e': 3}
+    tokens = {r: tokens_for(config, n, seed) for seed, (r, n) in enumerate(lengths.items())}
+    expected = {r: plain.logits(t, weights, config) for r, t in tokens.items()}
+    for r in lengths:
+        runner.admit(r)
+    # a, c and e have all but their last token behind them; b and d bring portions
+    runner.step([StepEntry(r, tuple(tokens[r][:-1]), ()) for r in 'ace'])
+    runner.step([StepEntry('b', tuple(tokens['b'][:4]), ()), StepEntry('d', tuple(tokens['d'][:2]), ())])
+    entries = [StepEntry('a', tuple(tokens['a'][-1:]), (0,)), StepEntry('b', tuple(tokens['b'][4:]), (7, 0, 3)),
+               StepEntry('c', tuple(tokens['c'][-1:]), ()), StepEntry('d', tuple(tokens['d'][2:]), (6,)),
+               StepEntry('e', tuple(tokens['e'][-1:]), (0,))]
+    described, ctx = runner.prepare(entries)
+    assert [e.request for e in described] == ['b', 'd', 'a', 'c', 'e'] == ctx.requests and ctx.tile_seqs == 2
+    assert ctx.single_rows.tolist() == [15, 16, 17] and ctx.logit_rows.tolist() == [15, 7, 0, 3, 14, 17]
+    logits = runner.step(entries)
+    want = torch.stack([expected['a'][6], expected['b'][11], expected['b'][4], expected['b'][7], expected['d'][8],
+                        expected['e'][2]])
+    case.close(logits, want)
+    assert all(runner.computed(r) == n for r, n in lengths.items())
+
+
 def test_step_validation(case):
     config, weights, model, page_size = case
     runner = ModelRunner(model, num_pages=2, page_size=page_size)
