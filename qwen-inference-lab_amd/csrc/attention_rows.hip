@@ -24,6 +24,17 @@
 #define ATT_THREADS 256
 #define ATT_WAVES (ATT_THREADS / QIL_WAVE)
 
+// The sum of every 16 consecutive lanes, in their first lane (all lanes get a sum of the 16 values; the order of the
+// additions is the first lane's in every group).  Four data-parallel moves: neighbours, pairs, fours mirrored in
+// a half row, eights mirrored in the row.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+  return v;
+}
+
 template <typename T, int GT>
 __global__ void __launch_bounds__(ATT_THREADS)
 attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
@@ -114,47 +125,54 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
     }
     __syncthreads();
 
-    // ---- weighted values
-    float acc[GT][8];
-#pragma unroll
-    for (int h = 0; h < GT; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-    for (int t0 = wave * TPW + slot; t0 < count; t0 += 4 * stride) {      // four keys at a time, as above
-      float vv[4][8];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int j = begin + min(t0 + u * stride, count - 1);
-        const size_t page = table[j / page_size];
-        // V is [pages, kv_heads, d, page_size]: this key's elements lie page_size apart
-        const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + e0) * page_size + (j % page_size);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) vv[u][e] = live ? ld(column + (size_t)e * page_size) : 0.f;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int t = t0 + u * stride;
-        if (t < count) {
-#pragma unroll
-          for (int h = 0; h < GT; ++h) {
-            const float p = scores[h * P + t];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] += p * vv[u][e];
-          }
-        }
-      }
-    }
-    // sum over the token slots of the wave, then over the waves (fixed order)
-#pragma unroll
-    for (int h = 0; h < GT; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        for (int o = TG; o < QIL_WAVE; o <<= 1) acc[h][e] += __shfl_xor(acc[h][e], o, QIL_WAVE);
-    if (slot == 0 && live) {
+    // ---- weighted values.  V is [pages, kv_heads, d, page_size]: a key's elements lie page_size apart and the keys
+    // of a page side by side, so here a wave's lanes are 16 consecutive keys x 4 chunks of 8 elements (a load
+    // instruction then reads whole 64-byte runs of 16 keys, not 16 bytes of 4 keys), and the head's elements are
+    // taken 32 at a time.
+    const int v_key = lane & 15, v_e0 = (lane >> 4) * 8;
+    for (int c0 = 0; c0 < d; c0 += 32) {
+      const int ve = c0 + v_e0;
+      const bool v_live = ve < d;
+      float acc[GT][8];
 #pragma unroll
       for (int h = 0; h < GT; ++h)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) wave_acc[(wave * GT + h) * d + e0 + e] = acc[h][e];
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
+      constexpr int V_STRIDE = ATT_WAVES * 16;
+      for (int t0 = wave * 16 + v_key; t0 < count; t0 += 2 * V_STRIDE) {      // two keys at a time, their loads first
+        float vv[2][8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int j = begin + min(t0 + u * V_STRIDE, count - 1);
+          const size_t page = table[j / page_size];
+          const T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + ve) * page_size + (j % page_size);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vv[u][e] = v_live ? ld(column + (size_t)e * page_size) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int t = t0 + u * V_STRIDE;
+          if (t < count) {
+#pragma unroll
+            for (int h = 0; h < GT; ++h) {
+              const float p = scores[h * P + t];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) acc[h][e] += p * vv[u][e];
+            }
+          }
+        }
+      }
+      // sum over the wave's 16 keys (fixed order), then over the waves below
+#pragma unroll
+      for (int h = 0; h < GT; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] = row16_sum(acc[h][e]);
+      if (v_key == 0 && v_live) {
+#pragma unroll
+        for (int h = 0; h < GT; ++h)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) wave_acc[(wave * GT + h) * d + ve + e] = acc[h][e];
+      }
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < GT * d; idx += ATT_THREADS) {

@@ -28,10 +28,11 @@ STREAM_GEMM_MOST_ROWS = 192
 # it is ahead from 17 rows on, without it level with the staged kernel up to 32 rows.
 MID_GEMM_FEWEST_ROWS, MID_GEMM_MOST_ROWS = 33, 256
 MID_GATED_FEWEST_ROWS = 17
-# Keys per split of the row attention kernel at 8 rows of 2,048 keys; _rows_part scales it with the work.
+# Half the most keys a split of the row attention kernel gets (_rows_part scales the split with the work); tests set
+# another value to force it.
 ATTENTION_PART = 256
 # Blocks the row attention kernel aims for.
-ROWS_BLOCKS = 512
+ROWS_BLOCKS = 1024
 # Blocks the matrix-core decode kernel aims for (256 CUs, 8 waves a block; measured best at 8 rows x 2048 keys).
 DECODE_BLOCKS = 256
 # Waves of a block of that kernel; each takes every DECODE_WAVES-th 32-key step of the block's keys.
@@ -414,8 +415,9 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 def _rows_part(rows, kv_heads, max_context):
     """Keys a part of the row kernel: about ROWS_BLOCKS blocks in all, parts of 64 to ATTENTION_PART * 2 keys
-    (measured in float32 at 2,048 keys of 8 kv heads: 1 row 36 us with parts of 64 against 54 with 256; 8 rows
-    best at 256; 64 rows best at 512)."""
+    (measured in float32 at 2,048 keys of 8 kv heads: 1 row 28 us with parts of 64 to 256 against 67 with 512;
+    8 rows 45 us with 128 against 54 with 256 and 62 with 64; 64 rows level from 256 on; 8 rows of 8,192 keys best
+    at 256 and 512)."""
     if ATTENTION_PART != 256:                          # a test or tuning run has set it
         return ATTENTION_PART
     wanted = max_context * rows * kv_heads / ROWS_BLOCKS

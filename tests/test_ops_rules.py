@@ -3,12 +3,13 @@ from qil_amd import ops
 
 
 def test_row_kernel_parts_scale_with_the_work():
-    """One row of 2,048 keys is cut into parts of 64 keys, eight rows into parts of 256, sixty-four into parts of
+    """One row of 2,048 keys is cut into parts of 64 keys, eight rows into parts of 128, sixty-four into parts of
     512; never below 64 or above 512, and a power of two."""
     kv_heads = 8
     assert ops._rows_part(1, kv_heads, 2048) == 64
-    assert ops._rows_part(8, kv_heads, 2048) == 256
-    assert ops._rows_part(8, kv_heads, 2100) == 256
+    assert ops._rows_part(8, kv_heads, 2048) == 128
+    assert ops._rows_part(8, kv_heads, 2100) == 128
+    assert ops._rows_part(8, kv_heads, 8192) == 512
     assert ops._rows_part(64, kv_heads, 2048) == 512
     assert ops._rows_part(1, 1, 5) == 64
     assert ops._rows_part(128, 8, 100000) == 512
