@@ -315,6 +315,10 @@ extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
   return sp < 1 ? 1 : sp;
 }
 
+extern "C" int qil_gemm_f32_mfma_takes(int M, int N, int K);                  // gemm_f32_mfma.hip
+extern "C" int qil_gemm_f32_mfma(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
+                                 hipStream_t s);
+
 // C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs M <= 64,
 // K % 4 == 0 and no bias.
 extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
@@ -358,6 +362,14 @@ extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, f
                          M, N, K, m0);
     QIL_RETURN_LAUNCH_STATUS();
   }
+  // many rows: the matrix-core kernel where it takes the sizes (K in whole stages of 32, aligned operands) and its
+  // blocks of 256 x 128 results fill most of the chip; a block runs through all of K at 3.9 us a stage, so with few
+  // blocks the small tiles below are faster (measured at K = 4,096: 1,024 x 6,144 in 192 blocks 546 against 755 us,
+  // 512 x 6,144 in 96 blocks 522 against 420; 128 rows, half a tile: 533 against 416 in 192 blocks)
+  const long mfma_blocks = (long)((M + 255) / 256) * ((N + 127) / 128);
+  if (M > 128 && mfma_blocks >= 160 && qil_gemm_f32_mfma_takes(M, N, K) &&
+      (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) % 16) == 0)
+    return qil_gemm_f32_mfma(A, W, bias, C, M, N, K, s);
   dim3 grid((N + SG_BN - 1) / SG_BN, (M + SG_BM - 1) / SG_BM);
   const bool vec = (K % 4 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
   if (vec) hipLaunchKernelGGL(sgemm_nt_kernel<true>, grid, dim3(256), 0, s, A, W, bias, C, M, N, K);

@@ -143,6 +143,33 @@ def test_linear_float32_partial_sums(ops, m, n, k):
         assert isinstance(got, ops.Partials), 'a product with few columns and a long K should be split'
 
 
+@pytest.mark.parametrize('m', [65, 255, 256, 257, 700])
+@pytest.mark.parametrize('n,k', [(128, 64), (130, 96), (97, 4096), (1000, 224), (6144, 1024)])
+def test_linear_float32_of_many_rows_on_the_matrix_cores(ops, m, n, k):
+    """The float32 product of more than 64 rows with K in whole stages of 32: v_mfma_f32_32x32x2_f32 on tiles loaded
+    straight into LDS.  Row and column counts that end inside a block's 256 x 128 tile, inside a wave's tile and
+    inside a group of four columns; 2 stages (the fewest) to 128; with and without bias; against float64.  A row's
+    result is the same in another place of another batch, bit for bit."""
+    lib = ops.library.load()
+    x, w, b = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5), rand(n, seed=2)
+    want = x.double() @ w.double().t()
+    assert lib.qil_gemm_f32_mfma_takes(m, n, k) and not lib.qil_gemm_f32_mfma_takes(m, n, k + 16)
+    raw = torch.cuda.current_stream().cuda_stream
+    # a sum of 4,096 float32 products made one after the other is further from float64 than one of 1,024 (measured
+    # on these numbers: 9.6e-6 at most here, 1.07e-5 by the vector units' kernel at K = 4,100, which adds the same way)
+    scale = 4 if k < 4096 else 8
+    def product(rows, bias):
+        out = torch.full((rows.shape[0], n), float('nan'), device='cuda')
+        assert lib.qil_gemm_f32_mfma(rows.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                     out.data_ptr(), rows.shape[0], n, k, raw) == 0
+        return out
+    check(product(x, None), want, torch.float32, scale=scale)
+    check(product(x, b), want + b.double(), torch.float32, scale=scale)
+    moved = torch.cat([x[m - 60:], x[:3]]).contiguous()
+    torch.testing.assert_close(product(moved, None)[:60], product(x, None)[m - 60:], atol=0, rtol=0)
+    check(ops.linear(x, w, b), want + b.double(), torch.float32, scale=scale)    # the op, whichever kernel it picks
+
+
 @pytest.mark.parametrize('m,n,k', SHAPES)
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('bias', [False, True])
