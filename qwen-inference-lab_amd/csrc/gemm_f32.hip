@@ -6,6 +6,8 @@
 // kernel below (float32 matrix-core instruction, still no reduced-precision input).  Both operands
 // have K contiguous (nn.Linear layout, qil/model.py:32-40).  The tiled kernel: 64 x 64 x 16 tiles in
 // LDS, 256 threads, 4 x 4 outputs a thread.
+#include <algorithm>
+
 #include "common.h"
 
 #define SG_BM 64
@@ -304,9 +306,32 @@ static int fl_splits(int M, int N, int K) {
   return fit;
 }
 
-// Ways the few-row product will be split over K when partial sums are allowed (1: it is not split).
+extern "C" int qil_gemm_f32_mfma_takes(int M, int N, int K, int splits);      // gemm_f32_mfma.hip
+extern "C" long qil_gemm_f32_mfma_blocks(int M, int N);
+extern "C" int qil_gemm_f32_mfma_splits(int M, int N, int K);
+extern "C" int qil_gemm_f32_mfma(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
+                                 int splits, hipStream_t s);
+
+// More than 64 rows: the matrix-core kernel where it takes the sizes (K in whole stages of 32) and is the faster one
+// by this count.  A block of the matrix-core kernel runs through its part of K at 3.9 us a stage (2.0 with 128 rows),
+// one block a CU; the vector units' kernel takes 0.069 us a column of K however few rows there are and reaches 61 to
+// 74 TFLOP/s with many.  Measured at K = 4,096 unsplit: 1,024 x 6,144 in 192 blocks 546 against 755 us, 512 x 6,144 in
+// 96 blocks 522 against 420; in two splits 276.
+static bool mfma_wanted(int M, int N, int K, int splits) {
+  if (M <= SF_MOST_ROWS || !qil_gemm_f32_mfma_takes(M, N, K, splits)) return false;
+  const double rounds = (double)((qil_gemm_f32_mfma_blocks(M, N) * splits + 255) / 256);
+  const double matrix = rounds * (K / 32 / splits) * (M <= 128 ? 2.0 : 3.9) + 8.0;
+  const double vector = std::max(0.069 * K, 2.0 * ((M + 63) / 64 * 64) * N * (double)K / 66e6);   // 64-row tiles, 61 to 74 TFLOP/s
+  return matrix < vector;
+}
+
+// Ways the product will be split over K when partial sums are allowed (1: it is not split).
 extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
-  if (M > SF_MOST_ROWS || K % 4) return 1;
+  if (M > SF_MOST_ROWS) {
+    const int sp = qil_gemm_f32_mfma_splits(M, N, K);
+    return mfma_wanted(M, N, K, sp) ? sp : 1;
+  }
+  if (K % 4) return 1;
   if (const int lines = fl_splits(M, N, K)) return lines;
   const int column_blocks = (N + 127) / 128, steps = (K + 15) / 16;
   int sp = (768 + column_blocks - 1) / column_blocks;
@@ -315,17 +340,16 @@ extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
   return sp < 1 ? 1 : sp;
 }
 
-extern "C" int qil_gemm_f32_mfma_takes(int M, int N, int K);                  // gemm_f32_mfma.hip
-extern "C" int qil_gemm_f32_mfma(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
-                                 hipStream_t s);
-
-// C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs M <= 64,
-// K % 4 == 0 and no bias.
+// C float32 [splits, M, N] (the value is the sum over the first axis); splits > 1 needs no bias and either M <= 64
+// and K % 4 == 0, or the number of splits that qil_gemm_f32_splits gives for more rows.
 extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, float* C, int M, int N, int K,
                             int splits, hipStream_t s) {
   if (M == 0 || N == 0) return 0;
   if (K < 1 || splits < 1) return -1;
   const bool stream_ok = M <= SF_MOST_ROWS && K % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
+  if (M > SF_MOST_ROWS && mfma_wanted(M, N, K, splits) && !(bias && splits > 1) &&
+      (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) % 16) == 0)
+    return qil_gemm_f32_mfma(A, W, bias, C, M, N, K, splits, s);
   if (splits > 1 && (!stream_ok || bias)) return -1;
   if (stream_ok && !bias && splits == fl_splits(M, N, K) && fl_takes(M, N, K, splits)) {
     const size_t lds = fl_lds_bytes(M, K, splits);
@@ -362,14 +386,6 @@ extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, f
                          M, N, K, m0);
     QIL_RETURN_LAUNCH_STATUS();
   }
-  // many rows: the matrix-core kernel where it takes the sizes (K in whole stages of 32, aligned operands) and its
-  // blocks of 256 x 128 results fill most of the chip; a block runs through all of K at 3.9 us a stage, so with few
-  // blocks the small tiles below are faster (measured at K = 4,096: 1,024 x 6,144 in 192 blocks 546 against 755 us,
-  // 512 x 6,144 in 96 blocks 522 against 420; 128 rows, half a tile: 533 against 416 in 192 blocks)
-  const long mfma_blocks = (long)((M + 255) / 256) * ((N + 127) / 128);
-  if (M > 128 && mfma_blocks >= 160 && qil_gemm_f32_mfma_takes(M, N, K) &&
-      (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) % 16) == 0)
-    return qil_gemm_f32_mfma(A, W, bias, C, M, N, K, s);
   dim3 grid((N + SG_BN - 1) / SG_BN, (M + SG_BM - 1) / SG_BM);
   const bool vec = (K % 4 == 0) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
   if (vec) hipLaunchKernelGGL(sgemm_nt_kernel<true>, grid, dim3(256), 0, s, A, W, bias, C, M, N, K);

@@ -155,8 +155,10 @@ def _declare(lib):
     lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_splits.argtypes = [i, i, i]
-    lib.qil_gemm_f32_mfma.argtypes = [p, p, p, p, i, i, i, p]
-    lib.qil_gemm_f32_mfma_takes.argtypes = [i, i, i]
+    lib.qil_gemm_f32_mfma.argtypes = [p, p, p, p, i, i, i, i, p]
+    lib.qil_gemm_f32_mfma_takes.argtypes = [i, i, i, i]
+    lib.qil_gemm_f32_mfma_splits.argtypes = [i, i, i]
+    lib.qil_gemm_f32_mfma_splits.restype = i
     lib.qil_gemm_f32_mfma_takes.restype = i
     lib.qil_gemm_f32_splits.restype = i
     lib.qil_gemm_bf16.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]

@@ -126,15 +126,15 @@ def test_linear_float32_whole_lines(ops, m, k):
 
 
 @pytest.mark.parametrize('m,n,k', [(3, 1024, 4096), (16, 300, 2048), (20, 4096, 4096), (64, 1024, 3072), (33, 130, 516),
-                                   (48, 2000, 100), (65, 512, 1024)])
+                                   (48, 2000, 100), (65, 512, 1024), (128, 4096, 1024), (160, 6144, 4096)])
 def test_linear_float32_partial_sums(ops, m, n, k):
     """Up to 64 rows the float32 product streams W through the float32 matrix-core instruction and may come
-    back split over K; with more rows it is one tensor."""
+    back split over K; with more rows it is one tensor unless the tiled matrix-core kernel splits K to fill the chip."""
     x, w = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5)
     got = ops.linear(x, w, None, partials=True)
     want = x.double() @ w.double().t()
     if isinstance(got, ops.Partials):
-        assert m <= 64 and got.splits > 1 and got.shape == (m, n)
+        assert got.splits == ops.library.load().qil_gemm_f32_splits(m, n, k) > 1 and got.shape == (m, n)
         check(got.sum(), want, torch.float32, scale=4)
     else:
         assert m > 64 or ops.library.load().qil_gemm_f32_splits(m, n, k) == 1
@@ -143,31 +143,47 @@ def test_linear_float32_partial_sums(ops, m, n, k):
         assert isinstance(got, ops.Partials), 'a product with few columns and a long K should be split'
 
 
-@pytest.mark.parametrize('m', [65, 255, 256, 257, 700])
+@pytest.mark.parametrize('m', [65, 127, 128, 129, 255, 256, 257, 700])
 @pytest.mark.parametrize('n,k', [(128, 64), (130, 96), (97, 4096), (1000, 224), (6144, 1024)])
 def test_linear_float32_of_many_rows_on_the_matrix_cores(ops, m, n, k):
     """The float32 product of more than 64 rows with K in whole stages of 32: v_mfma_f32_32x32x2_f32 on tiles loaded
-    straight into LDS.  Row and column counts that end inside a block's 256 x 128 tile, inside a wave's tile and
-    inside a group of four columns; 2 stages (the fewest) to 128; with and without bias; against float64.  A row's
-    result is the same in another place of another batch, bit for bit."""
+    straight into LDS, 128 rows a block up to 128 rows and 256 beyond.  Row and column counts that end inside a
+    block's tile, inside a wave's tile and inside a group of four columns; 2 stages (the fewest) to 128; with and
+    without bias; K whole and in every number of splits it takes up to 8; against float64.  A row's result is the
+    same in another place of another batch, bit for bit."""
     lib = ops.library.load()
     x, w, b = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5), rand(n, seed=2)
     want = x.double() @ w.double().t()
-    assert lib.qil_gemm_f32_mfma_takes(m, n, k) and not lib.qil_gemm_f32_mfma_takes(m, n, k + 16)
+    assert lib.qil_gemm_f32_mfma_takes(m, n, k, 1) and not lib.qil_gemm_f32_mfma_takes(m, n, k + 16, 1)
     raw = torch.cuda.current_stream().cuda_stream
     # a sum of 4,096 float32 products made one after the other is further from float64 than one of 1,024 (measured
     # on these numbers: 9.6e-6 at most here, 1.07e-5 by the vector units' kernel at K = 4,100, which adds the same way)
     scale = 4 if k < 4096 else 8
-    def product(rows, bias):
-        out = torch.full((rows.shape[0], n), float('nan'), device='cuda')
-        assert lib.qil_gemm_f32_mfma(rows.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None,
-                                     out.data_ptr(), rows.shape[0], n, k, raw) == 0
-        return out
-    check(product(x, None), want, torch.float32, scale=scale)
-    check(product(x, b), want + b.double(), torch.float32, scale=scale)
+    def product(rows, bias, splits=1):
+        out = torch.full((splits, rows.shape[0], n), float('nan'), device='cuda')
+        status = lib.qil_gemm_f32_mfma(rows.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                       out.data_ptr(), rows.shape[0], n, k, splits, raw)
+        return status, out
+    status, whole = product(x, None)
+    assert status == 0
+    check(whole[0], want, torch.float32, scale=scale)
+    check(product(x, b)[1][0], want + b.double(), torch.float32, scale=scale)
     moved = torch.cat([x[m - 60:], x[:3]]).contiguous()
-    torch.testing.assert_close(product(moved, None)[:60], product(x, None)[m - 60:], atol=0, rtol=0)
+    torch.testing.assert_close(product(moved, None)[1][0, :60], whole[0, m - 60:], atol=0, rtol=0)
+    for splits in range(2, 9):
+        takes = (k // 32) % splits == 0 and k // 32 // splits >= 2
+        assert bool(lib.qil_gemm_f32_mfma_takes(m, n, k, splits)) == takes
+        status, parts = product(x, None, splits)
+        assert status == (0 if takes else -1)
+        if takes:
+            assert torch.isfinite(parts).all()
+            check(parts.double().sum(0), want, torch.float32, scale=scale)
+            assert product(x, b, splits)[0] == -1                                # a bias goes with one split
+    planned = lib.qil_gemm_f32_mfma_splits(m, n, k)
+    assert planned >= 1 and lib.qil_gemm_f32_mfma_takes(m, n, k, planned)
     check(ops.linear(x, w, b), want + b.double(), torch.float32, scale=scale)    # the op, whichever kernel it picks
+    got = ops.linear(x, w, None, partials=True)
+    check(got.sum() if isinstance(got, ops.Partials) else got, want, torch.float32, scale=scale)
 
 
 @pytest.mark.parametrize('m,n,k', SHAPES)
