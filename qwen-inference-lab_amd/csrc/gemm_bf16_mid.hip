@@ -7,8 +7,10 @@
 //    bytes for the same work).
 //  * W and A go from memory straight into LDS (global_load_lds_dwordx4, whole 128-byte lines, no registers): W into
 //    a ring of the wave's own, A into a ring that the block's multiplying waves share and a wave of its own fills
-//    (one barrier a stage of 64 columns of K).  Piece p of row r holds the columns 8 (p ^ (r & 7)) ..: fragment
-//    reads spread over the banks.
+//    (one barrier a stage of 64 columns of K).  Place p of row r holds the columns 8 (p ^ ((r >> 1) & 7)) ..: a
+//    fragment read takes 16 rows at a time, and rows two apart lie 256 bytes apart, on the same banks; with the
+//    place turned by r / 2 the 16 rows' pieces fall on all 64 banks once (turned by r, as at first, on half of
+//    them twice: the LDS counters showed every read taking twice its time).
 //  * A block is 2 to 4 multiplying waves (64 to 128 columns) and K is split over blocks, so that the blocks fill
 //    whole rounds of the 256 CUs (a block holds a CU's LDS); float32 partial sums [split][M][N] are added by the
 //    kernel that consumes them, as those of the few-row products are.  With one split the result is written in the
@@ -66,15 +68,16 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
   // eighth, at the same one, so that its L2 holds one band of A): they then read different columns of K and not all
   // the same narrow band of every row of W, which memory serves more slowly.
   const int turned = (int)((blockIdx.x % (unsigned)turns) * stages / turns);
-  // loads: a load is 8 rows of 128 bytes; lane = (row lane / 8, place lane % 8), and place p of row r takes piece p ^ (r & 7)
+  // loads: a load is 8 rows of 128 bytes; lane = (row lane / 8, place lane % 8), and place p of row r takes piece
+  // p ^ ((r >> 1) & 7): with r = 8 i + lane / 8 that is p ^ (lane / 16) in loads of even i and p ^ (lane / 16 + 4) in odd ones
   const int rl = lane >> 3;
-  const uint32_t piece_bytes = ((lane & 7) ^ rl) << 4;
+  const uint32_t piece_bytes[2] = {(uint32_t)((lane & 7) ^ (rl >> 1)) << 4, (uint32_t)((lane & 7) ^ ((rl >> 1) + 4)) << 4};
 
   if (wave == waves) {                                     // ---- the wave that loads A (the last of the block)
-    const char* a_from = reinterpret_cast<const char*>(A + k_begin) + piece_bytes;
+    const char* a_from = reinterpret_cast<const char*>(A + k_begin);
     uint32_t a_row_bytes[4 * MT];                          // rows past the last read it again: their results are not stored
 #pragma unroll
-    for (int j = 0; j < 4 * MT; ++j) a_row_bytes[j] = (uint32_t)min(8 * j + rl, M - 1) * (uint32_t)K * 2;
+    for (int j = 0; j < 4 * MT; ++j) a_row_bytes[j] = (uint32_t)min(8 * j + rl, M - 1) * (uint32_t)K * 2 + piece_bytes[j & 1];
     auto load_a = [&](int stage) __attribute__((always_inline)) {
       const int k_stage = stage + turned < stages ? stage + turned : stage + turned - stages;
       const size_t at = (size_t)k_stage * (MID_STAGE * 2);
@@ -102,7 +105,7 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
   const int l32 = lane & 31, half = lane >> 5;
   const int n0 = (blockIdx.x * waves + wave) * 32;         // the wave's columns (a wave past the end repeats the last ones)
   const int n_load = min(n0, N - 32);
-  const char* w_from = reinterpret_cast<const char*>(W + (size_t)(n_load + rl) * K + k_begin) + piece_bytes;
+  const char* w_from = reinterpret_cast<const char*>(W + (size_t)(n_load + rl) * K + k_begin);
   const size_t w_rows8 = (size_t)8 * K * 2;
   auto load_w = [&](int stage) __attribute__((always_inline)) {
     const int k_stage = stage + turned < stages ? stage + turned : stage + turned - stages;
@@ -110,11 +113,11 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
     unsigned char* w_to = lds + (stage % RW) * W_SLOT + wave * 4096;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_from + at + i * w_rows8),
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_from + at + i * w_rows8 + piece_bytes[i & 1]),
                                        (__attribute__((address_space(3))) void*)(w_to + i * 1024), 16, 0, 0);
   };
-  // fragment reads: lane = (row lane % 32, half lane / 32) wants piece 2 ks + half of its row: at place (2 ks) ^ (half ^ (row & 7))
-  const uint32_t piece = half ^ (l32 & 7);
+  // fragment reads: lane = (row lane % 32, half lane / 32) wants piece 2 ks + half of its row: at place (2 ks) ^ (half ^ ((row >> 1) & 7))
+  const uint32_t piece = half ^ ((l32 >> 1) & 7);
   uint32_t read_at[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) read_at[ks] = l32 * 128 + (((2 * ks) ^ piece) << 4);

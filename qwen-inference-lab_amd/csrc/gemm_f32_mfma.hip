@@ -8,8 +8,9 @@
 //  * K may be split over blocks (partial sums [split][M][N] that the consuming kernel adds in split order), for
 //    products whose tiles alone would leave most of the chip idle.
 //  * A stage is 32 columns of K: 256 rows of A and 128 rows of W, 128 bytes each, loaded straight from memory into
-//    LDS (global_load_lds_dwordx4: a wave's instruction takes 8 rows), piece p of row r at place p ^ (r & 7) so that
-//    the fragment reads spread over the banks.  Three stages lie in LDS; one barrier a stage.
+//    LDS (global_load_lds_dwordx4: a wave's instruction takes 8 rows), piece p of row r at place p ^ ((r >> 1) & 7):
+//    a fragment read takes 16 rows at a time, rows two apart lie on the same banks, and turned by r / 2 the 16 rows'
+//    pieces fall on all 64 banks once.  Three stages lie in LDS; one barrier a stage.
 //  * Loading and multiplying are different waves' work because of the compiler: it makes a wave that has sent a load
 //    into LDS wait for ALL its loads before its next LDS read, which would end the overlap of a stage's loads with the
 //    stage before.  A wave that only reads LDS, or only loads into it, gets no such wait.
@@ -32,11 +33,12 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 template <int COUNT, int SLOT>
 __device__ __forceinline__ void fm_load_loop(const float* source, int first, int last, int K, int stages,
                                              unsigned char* lds, uint32_t to, int lane) {
-  const int rl = lane >> 3;                                // lane = (row lane / 8, place lane % 8), which gets piece place ^ row
+  const int rl = lane >> 3;                                // lane = (row lane / 8, place lane % 8), which gets piece place ^ (row / 2 % 8)
   const char* from[COUNT];
 #pragma unroll
   for (int i = 0; i < COUNT; ++i)
-    from[i] = reinterpret_cast<const char*>(source + (size_t)min(first + 8 * i + rl, last) * K) + (((lane & 7) ^ rl) << 4);
+    from[i] = reinterpret_cast<const char*>(source + (size_t)min(first + 8 * i + rl, last) * K) +
+              (((lane & 7) ^ ((4 * i + (rl >> 1)) & 7)) << 4);
   auto load = [&](int stage) __attribute__((always_inline)) {
     unsigned char* slot = lds + (stage % FM_RING) * SLOT + to;
     const size_t at = (size_t)stage * (FM_STAGE * 4);
@@ -84,9 +86,9 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ W, c
   // ---- the waves that multiply: rows 64 (wave / 2) .. of A's tile, rows 64 (wave % 2) .. of W's
   const int l32 = lane & 31, half = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
-  uint32_t read_at[4];                                     // chunk c of this lane's row: piece 2 c + half, at place piece ^ (row & 7)
+  uint32_t read_at[4];                                     // chunk c of this lane's row: piece 2 c + half, at place piece ^ (row / 2 % 8)
 #pragma unroll
-  for (int c = 0; c < 4; ++c) read_at[c] = l32 * 128 + (((2 * c + half) ^ (l32 & 7)) << 4);
+  for (int c = 0; c < 4; ++c) read_at[c] = l32 * 128 + (((2 * c + half) ^ ((l32 >> 1) & 7)) << 4);
   const uint32_t a_rows = (wm * 64) * 128, w_rows = ROWS * 128 + (wn * 64) * 128;
 
   f32x16 acc[2][2];                                        // [tile of W's rows][tile of A's rows]
