@@ -2,7 +2,8 @@
 // all keys they see (qil/model.py:59-66 is the formula), keys and values loaded from memory straight into LDS.
 //
 // A block is 4 or 8 waves; a wave owns 32 rows of one head as ONE tile of v_mfma_f32_32x32x16_bf16, the waves of a
-// block are the heads of a kv group (and with 8 waves two row tiles): they share the staged keys.  Per tile of 64
+// block are the heads of a kv group (and with 8 waves two row tiles, or two groups that halve the keys): they share
+// the staged keys.  Per tile of 64
 // keys: S^T = K Q^T (16 products), softmax statistics in float32 registers, O^T += V^T P^T (16 products).
 //
 // A wave issues one instruction every four cycles and a product keeps the matrix core for 32, so what a tile costs
@@ -44,7 +45,12 @@ __device__ __forceinline__ int prompt_row(int kl) {
   return (kl & ~15) + ((kl >> 2) & 1) * 8 + ((kl >> 3) & 1) * 4 + (kl & 3);
 }
 
-template <int WAVES>
+// SPLIT (8 waves, no window, keys in one part): the block's waves are two groups of four that take the same rows and
+// heads and each one half of the block's tiles of keys, with two tiles in LDS of its own; at the end the second
+// group hands its sums over in LDS and the first adds them to its own.  For prompts so short that blocks of 4 waves
+// are fewer than the CUs: every SIMD then has two waves.  (It does not help longer prompts: a wave-tile takes 1.75 us
+// of its SIMD's issue slots whether the wave is alone there or not, and 2,048 tokens are 33 wave-tiles a SIMD.)
+template <int WAVES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES * QIL_WAVE, WAVES == 4 ? 2 : 1)
 attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
@@ -53,10 +59,11 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
                    float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P,
                    int parts) {
   constexpr int D = PROMPT_D, BK = PROMPT_BK, THREADS = WAVES * QIL_WAVE;
+  constexpr int GW = SPLIT ? WAVES / 2 : WAVES;            // waves that share a tile of keys
   constexpr int WFRAGS = D / 16, WTILES = D / 32;
-  constexpr int LOADS = 16 / WAVES;                        // K loads a wave and tile, and as many V loads
-  extern __shared__ __align__(1024) unsigned char lds[];   // two tiles (K then V each), then the table entries
-  int* pages = reinterpret_cast<int*>(lds + 2 * PROMPT_TILE_BYTES);
+  constexpr int LOADS = 16 / GW;                           // K loads a wave and tile, and as many V loads
+  extern __shared__ __align__(1024) unsigned char lds[];   // two tiles (K then V each) a group, then the table entries
+  int* pages = reinterpret_cast<int*>(lds + (SPLIT ? 4 : 2) * PROMPT_TILE_BYTES);
 
   // Which sequence, row tile and (kv head, head chunk) this block takes.  Blocks go to the 8 XCDs in turn, each
   // with an L2 of its own: when 256 is a multiple of the number of (sequence, kv head, chunk) triples, block id
@@ -83,14 +90,16 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   pair -= part * (kv_heads * chunks);
   const int q0 = cu_seqlens[seq], n = cu_seqlens[seq + 1] - q0;
   if (n < 2) return;
-  const int RT = WAVES / GH;
+  const int RT = GW / GH;
   const int block_rows = 32 * RT;
   const int tile_row0 = across * block_rows;
   if (tile_row0 >= n) return;
   const int kvh = pair / chunks, chunk = pair % chunks;
   const int g = heads / kv_heads;
   const int lane = threadIdx.x & (QIL_WAVE - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / QIL_WAVE);
+  const int block_wave = __builtin_amdgcn_readfirstlane(threadIdx.x / QIL_WAVE);
+  const int group = SPLIT ? block_wave / GW : 0, wave = SPLIT ? block_wave % GW : block_wave;   // wave: within its group
+  unsigned char* tiles = lds + group * 2 * PROMPT_TILE_BYTES;
   const int head_local = chunk * GH + wave % GH, row_group = wave / GH;
   const int wave_row0 = tile_row0 + row_group * 32;
   const bool wave_active = head_local < g && wave_row0 < n;
@@ -145,7 +154,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
 #pragma unroll
     for (int i = 0; i < 16; ++i) ow[t][i] = 0.f;
 
-  // ---- loads.  Load j = it * WAVES + wave of a tile: K keys 4 j .. 4 j + 3 (rows prompt_row(4 j) .. + 3, 1 KB), and
+  // ---- loads.  Load j = it * GW + wave of a tile: K keys 4 j .. 4 j + 3 (rows prompt_row(4 j) .. + 3, 1 KB), and
   // V^T of the 64 dims 64 (j % 2) .. of the 8 keys from 8 (j / 2) on: both in the page of key 4 j.
   const int low_page = key_begin >> ps_shift;
   const char* k_head = reinterpret_cast<const char*>(k_cache + (size_t)kvh * page_size * D);
@@ -155,21 +164,21 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   const uint32_t k_lane = (lane >> 4) * (D * 2) + (((lane & 15) ^ swizzle) << 4);
   const uint32_t v_lane = lane * page_size * 2;
   // Lane `it` looks the page of the loads `it` up, one tile ahead: `held` is in a register when it is needed.
-  const int held_key = (min(lane, LOADS - 1) * WAVES + wave) * 4;
+  const int held_key = (min(lane, LOADS - 1) * GW + wave) * 4;
   auto look_up = [&](int k0) __attribute__((always_inline)) {
     return pages[min(max((k0 + held_key) >> ps_shift, low_page), last_page) - first_page];
   };
   int held = 0;
   // One K or V load of tile k0 (in_page = k0 % page_size) into the tile at `to`.
   auto load_k = [&](int in_page, int it, unsigned char* to) __attribute__((always_inline)) {
-    const int key = (it * WAVES + wave) * 4;
+    const int key = (it * GW + wave) * 4;
     const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
     const uint32_t in = (uint32_t)(in_page + (key & (page_size - 1))) * (D * 2);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_head + page_at + in + k_lane),
                                      (__attribute__((address_space(3))) void*)(to + prompt_row(key) * (D * 2)), 16, 0, 0);
   };
   auto load_v = [&](int in_page, int it, unsigned char* to) __attribute__((always_inline)) {
-    const int j = it * WAVES + wave;
+    const int j = it * GW + wave;
     const size_t page_at = (size_t)(uint32_t)__builtin_amdgcn_readlane(held, it) << 8;
     const uint32_t in = (uint32_t)(in_page + ((j >> 1) * 8 & (page_size - 1))) * 2;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_head + page_at + in + v_lane),
@@ -186,7 +195,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   };
   // Values of keys outside [key_begin, key_end) of the tile at `tile` become zero (K needs none: the mask).
   auto zero_values = [&](int k0, unsigned char* tile) __attribute__((always_inline)) {
-    for (int idx = threadIdx.x; idx < BK / 8 * D; idx += THREADS) {
+    for (int idx = threadIdx.x % (GW * QIL_WAVE); idx < BK / 8 * D; idx += GW * QIL_WAVE) {
       const int key = k0 + idx / D * 8;
       if (key >= key_begin && key + 8 <= key_end) continue;
       uint4* cell = reinterpret_cast<uint4*>(tile + BK * D * 2) + idx;
@@ -307,9 +316,59 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   };
 
   __syncthreads();                                         // the table entries are in place
-  held = look_up(first_tile);
-  load_tile(first_tile, lds);
   int buffer = 0;
+  if constexpr (SPLIT) {
+    // The block's T tiles of keys: the first T / 2 to group 0, the others (the diagonal among them) to group 1.  Both
+    // groups make the same number of steps, with the same barriers; group 0 sits the last one out when T is odd.
+    const int T = (key_end - first_tile + BK - 1) / BK;
+    const int mine = group == 0 ? T / 2 : T - T / 2, steps = T - T / 2;
+    int k0 = first_tile + (group == 0 ? 0 : (T / 2) * BK);
+    held = look_up(k0);
+    load_tile(k0, tiles);
+    for (int step = 0; step < steps; ++step, k0 += BK) {
+      unsigned char* tile = tiles + buffer * PROMPT_TILE_BYTES;
+      unsigned char* next = tiles + (buffer ^ 1) * PROMPT_TILE_BYTES;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's loads of the tile have landed
+      __syncthreads();                                     // everyone's have, and everyone is done with the tile before
+      if (step == steps - 1) {                             // the last tile may hold keys past the sequence's end
+        if (step < mine && k0 + BK > key_end) zero_values(k0, tile);
+        __syncthreads();
+      }
+      if (step < mine && wave_active && k0 <= wave_last_pos) {
+        const bool all_visible = k0 + BK - 1 <= start + wave_row0 && wave_row0 + 32 <= n;
+        attend(k0, tile, next, !all_visible);
+      } else if (step + 1 < mine) {
+        load_tile(k0 + BK, next);
+      }
+      buffer ^= 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // no load into LDS is on its way
+    __syncthreads();                                       // and nobody reads a tile any more: their place takes the sums
+    // group 1's sums of a lane: 64 accumulators, the exponents' reference and the sum of probabilities, lane by lane
+    float* handed = reinterpret_cast<float*>(lds) + (size_t)wave * (WTILES * 16 + 2) * QIL_WAVE + lane;
+    if (group == 1) {
+#pragma unroll
+      for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) handed[(t * 16 + i) * QIL_WAVE] = ow[t][i];
+      handed[(WTILES * 16) * QIL_WAVE] = row_m;
+      handed[(WTILES * 16 + 1) * QIL_WAVE] = row_l;
+    }
+    __syncthreads();
+    if (group == 1) return;
+    const float other_m = handed[(WTILES * 16) * QIL_WAVE], other_l = handed[(WTILES * 16 + 1) * QIL_WAVE];
+    const float m = fmaxf(row_m, other_m);
+    const float mine_scale = row_m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((row_m - m) * c);
+    const float other_scale = other_m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((other_m - m) * c);
+#pragma unroll
+    for (int t = 0; t < WTILES; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ow[t][i] = ow[t][i] * mine_scale + handed[(t * 16 + i) * QIL_WAVE] * other_scale;
+    row_l = row_l * mine_scale + other_l * other_scale;
+    row_m = m;
+  } else {
+  held = look_up(first_tile);
+  load_tile(first_tile, tiles);
   auto tile_step = [&](int k0, auto edge_tag) __attribute__((always_inline)) {
     unsigned char* tile = lds + buffer * PROMPT_TILE_BYTES;
     unsigned char* next = lds + (buffer ^ 1) * PROMPT_TILE_BYTES;
@@ -334,6 +393,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
   for (k0 += BK; k0 + BK < key_end; k0 += BK) tile_step(k0, std::false_type());
   if (k0 < key_end) tile_step(k0, std::true_type());
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // no load into LDS is on its way when the block ends
+  }
 
   if (!wave_active) return;
   const float total = row_l + __shfl_xor(row_l, 32, QIL_WAVE);
@@ -364,15 +424,15 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
           make_uint2(pack_bf16(ow[t][4 * j] * inv, ow[t][4 * j + 1] * inv), pack_bf16(ow[t][4 * j + 2] * inv, ow[t][4 * j + 3] * inv));
 }
 
-template <int WAVES>
+template <int WAVES, bool SPLIT = false>
 static int launch_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                          int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                          int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s,
                          float* workspace, int total_rows, int P, int parts) {
   const int g = heads / kv_heads;
-  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = WAVES / GH;
-  const size_t lds = 2 * (size_t)PROMPT_TILE_BYTES + (size_t)table_stride * sizeof(int);
-  auto kernel = attn_prompt_kernel<WAVES>;
+  const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = (SPLIT ? WAVES / 2 : WAVES) / GH;
+  const size_t lds = (SPLIT ? 4 : 2) * (size_t)PROMPT_TILE_BYTES + (size_t)table_stride * sizeof(int);
+  auto kernel = attn_prompt_kernel<WAVES, SPLIT>;
   static size_t granted = 0;                     // per instantiation
   if (lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -398,7 +458,8 @@ extern "C" int qil_attn_prompt_takes(int d, int page_size, int table_stride) {
          table_stride <= PROMPT_TABLE_MAX;
 }
 
-// Sequences with two or more rows (the others' rows stay unwritten).  waves: 4 or 8 a block.  parts == 1: out
+// Sequences with two or more rows (the others' rows stay unwritten).  waves: 4 or 8 a block, or 16: 8 waves in two
+// groups that split a block's keys between them (no window, keys in one part).  parts == 1: out
 // [rows, heads * 128]; parts > 1: the keys in parts of P keys (a multiple of 64), float32 partial results in
 // `workspace` for the merge kernel, `out` unused.  The caller has checked the sizes (qil_attn_prompt_takes).
 extern "C" int qil_attn_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache,
@@ -407,9 +468,14 @@ extern "C" int qil_attn_prompt(const void* q, int q_stride, const void* k_cache,
                                float scale, int waves, void* workspace, int total_rows, int P, int parts, hipStream_t s) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (!qil_attn_prompt_takes(PROMPT_D, page_size, table_stride) || heads % kv_heads || n_seqs > 65535 ||
-      (long)kv_heads * 2 * parts > 65535 || (waves != 4 && waves != 8) || parts < 1 ||
+      (long)kv_heads * 2 * parts > 65535 || (waves != 4 && waves != 8 && waves != 16) || parts < 1 ||
+      (waves == 16 && (window > 0 || parts > 1)) ||
       (parts > 1 && (!workspace || total_rows < 1 || P < PROMPT_BK || P % PROMPT_BK)) || (parts == 1 && !out))
     return -1;
+  if (waves == 16)
+    return launch_prompt<8, true>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, s, (float*)workspace,
+                                  total_rows, P, parts);
   if (waves == 8)
     return launch_prompt<8>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
                             max_query, heads, kv_heads, page_size, window, scale, s, (float*)workspace, total_rows, P, parts);

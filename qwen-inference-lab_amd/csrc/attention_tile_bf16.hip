@@ -545,9 +545,14 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
     const int g128 = heads / kv_heads, gh128 = g128 >= 3 ? 4 : g128;
     const long blocks4 = (long)((max_query + 32 * (4 / gh128) - 1) / (32 * (4 / gh128))) * n_seqs * kv_heads *
                          ((g128 + gh128 - 1) / gh128);
-    const bool wide = tile_waves_override ? tile_waves_override == 8 : blocks4 >= 2048;
+    // Fewer blocks of 4 waves than CUs (one prompt of up to 1,024 tokens with 8 kv heads): 8 waves in two groups that
+    // split a block's keys, so that every SIMD has two waves (16 : 23 us at 256 tokens, 19 : 20 at 512, 27 : 29 at
+    // 1,024; with more blocks the SIMDs are full anyway and the merge at the end only costs: 66 : 57 at 2,048).
+    int waves = blocks4 >= 2048 ? 8 : blocks4 <= 256 && window <= 0 ? 16 : 4;
+    if (tile_waves_override) waves = tile_waves_override;   // 4, 8, or 16 (the two groups)
+    if (waves == 16 && window > 0) waves = 4;
     return qil_attn_prompt(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
-                           max_query, heads, kv_heads, page_size, window, scale, wide ? 8 : 4, nullptr, 0, 0, 1, s);
+                           max_query, heads, kv_heads, page_size, window, scale, waves, nullptr, 0, 0, 1, s);
   }
   return launch_fast<256, 1, 4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                 n_seqs, max_query, heads, kv_heads, page_size, window, scale, s);

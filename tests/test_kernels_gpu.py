@@ -751,7 +751,7 @@ def test_prompt_portions_against_float64(ops, dtype, lengths, chunks, page_size,
 
 
 @pytest.mark.parametrize('growth', [0.02, 0.11, 1.5])
-@pytest.mark.parametrize('waves', [4, 8])
+@pytest.mark.parametrize('waves', [4, 8, 16])
 def test_prompt_attention_with_scores_that_grow_along_the_keys(ops, growth, waves):
     """The kernel for head size 128 keeps a row's reference exponent until a score exceeds it by 2^8.  Keys whose
     scores grow by `growth` (in the exponent, to base 2) from one key to the next move it never within a tile's
