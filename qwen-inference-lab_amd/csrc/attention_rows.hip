@@ -200,7 +200,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
 }
 
 // One wave a block; a head takes tg lanes (a power of two >= d / 4, four elements a lane), 64 / tg heads a wave.
-// The parts are read four at a time with all their loads first; the sums run over the parts in order.
+// The parts are read eight at a time with all their loads first; the sums run over the parts in order.
 template <typename T>
 __global__ void __launch_bounds__(QIL_WAVE)
 attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
@@ -209,34 +209,37 @@ attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restri
                        int window, int P, int parts, int tg) {
   const int slot_row = blockIdx.x;
   const int head = blockIdx.y * (QIL_WAVE / tg) + threadIdx.x / tg, e = (threadIdx.x % tg) * 4;
-  if (head >= heads || e >= d) return;
+  const bool head_there = head < heads;                    // the same for the tg lanes of a head; all of them take part in the maximum
   const int row = row_index ? row_index[slot_row] : slot_row;
   const int ctx = positions[row] + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
   const int first = lo / P, last = (ctx - 1) / P;
   const size_t cell0 = ((size_t)slot_row * heads + head) * parts;
+  // the largest exponent: a head's lanes take a part each, then the largest among them (one round trip to memory for
+  // up to tg parts, not one for every four)
   float m = -INFINITY;
-  for (int p0 = first; p0 <= last; p0 += 4) {
-    float mv[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) mv[j] = part_m[cell0 + min(p0 + j, last)];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) m = fmaxf(m, mv[j]);
+  for (int p0 = first; p0 <= last; p0 += tg) {
+    const int p = p0 + (int)(threadIdx.x % tg);
+    if (head_there && p <= last) m = fmaxf(m, part_m[cell0 + p]);
   }
+  for (int o = tg >> 1; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, QIL_WAVE));
+  if (!head_there || e >= d) return;
+  // the sums run over the parts in order, eight parts' loads at a time
+  constexpr int AT_ONCE = 8;
   float denom = 0.f;
   float4 numer = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int p0 = first; p0 <= last; p0 += 4) {
-    float mv[4], lv[4];
-    float4 acc[4];
+  for (int p0 = first; p0 <= last; p0 += AT_ONCE) {
+    float mv[AT_ONCE], lv[AT_ONCE];
+    float4 acc[AT_ONCE];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < AT_ONCE; ++j) {
       const size_t cell = cell0 + min(p0 + j, last);
       mv[j] = part_m[cell];
       lv[j] = part_l[cell];
       acc[j] = *reinterpret_cast<const float4*>(part_acc + cell * d + e);
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < AT_ONCE; ++j) {
       if (p0 + j <= last) {
         const float f = expf(mv[j] - m);
         denom += lv[j] * f;
