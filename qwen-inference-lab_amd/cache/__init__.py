@@ -1,5 +1,5 @@
 """Cache: pages, block tables and state slots."""
 from .pages import PagePool, CacheFull
-from .manager import CacheManager, KVView, StateView
+from .manager import CacheManager, KVView, PagedView, StateView
 
-__all__ = ['PagePool', 'CacheFull', 'CacheManager', 'KVView', 'StateView']
+__all__ = ['PagePool', 'CacheFull', 'CacheManager', 'KVView', 'PagedView', 'StateView']

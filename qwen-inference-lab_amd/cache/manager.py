@@ -2,8 +2,8 @@
 slots for fixed-size per-request state, and the device storage behind them.
 
 Needs come from the model (``CausalLM.cache_needs()``), one per schedule entry.
-Entries with equal KV needs (kv heads, head size, window) form a group with a
-page pool of its own; every group has its own block tables, so a windowed group
+Entries with equal paged needs (``KVNeed``: kv heads, head size, window; or a ``PagedNeed`` with
+tensors of the mixer's own) form a group with a page pool of its own; every group has its own block tables, so a windowed group
 can give pages back while a full group keeps them.  Entries with equal state
 needs form a state group.  Device layout of a KV group:
 ``k : [entries, pages, kv_heads, page_size, head_dim]`` and, transposed within a page so
@@ -22,7 +22,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import KVNeed, StateNeed
+from ..parts.base import KVNeed, PagedNeed, StateNeed
 from .pages import PagePool, CacheFull
 
 
@@ -33,6 +33,17 @@ class KVView:
     v: torch.Tensor              # [pages, kv_heads, head_dim, page_size]
     page_size: int
     writes: bool                 # False for an entry that reads another entry's cache
+    group: int
+    block_tables: torch.Tensor = None    # int32 [n_seqs, stride], filled per step
+    slots: torch.Tensor = None           # int32 [n_tokens], slot of each new token
+
+
+@dataclass
+class PagedView:
+    """What a mixer with a ``PagedNeed`` sees of its schedule entry's cache in one step."""
+    tensors: dict                # name -> [pages, page_size, *shape of a token's entry]
+    page_size: int
+    writes: bool
     group: int
     block_tables: torch.Tensor = None    # int32 [n_seqs, stride], filled per step
     slots: torch.Tensor = None           # int32 [n_tokens], slot of each new token
@@ -58,7 +69,7 @@ class CacheManager:
             elif isinstance(need, tuple) and need[0] == 'shared':
                 kind, group, index, _ = self.binding[need[1]]
                 self.binding.append((kind, group, index, False))
-            elif isinstance(need, KVNeed):
+            elif isinstance(need, (KVNeed, PagedNeed)):
                 group = self._group(self.kv_groups, need)
                 self.binding.append(('kv', group, len(self.kv_groups[group]['entries']), True))
                 self.kv_groups[group]['entries'].append(position)
@@ -91,6 +102,12 @@ class CacheManager:
         for group in self.kv_groups:
             need, pool = group['need'], group['pool']
             entries, pages = len(group['entries']), pool.capacity
+            if isinstance(need, PagedNeed):
+                group['tensors'] = {
+                    name: torch.empty((entries, pages, self.page_size, *shape),
+                                      dtype=torch.float32 if kind == 'float32' else self.dtype, device=self.device)
+                    for name, shape, kind in need.tensors}
+                continue
             group['k'] = torch.empty((entries, pages, need.kv_heads, self.page_size, need.head_dim),
                                      dtype=self.dtype, device=self.device)
             group['v'] = torch.empty((entries, pages, need.kv_heads, need.head_dim, self.page_size),
@@ -188,11 +205,29 @@ class CacheManager:
             kind, group, index, writes = bound
             if kind == 'kv':
                 g = self.kv_groups[group]
-                out.append(KVView(g['k'][index], g['v'][index], self.page_size, writes, group))
+                if isinstance(g['need'], PagedNeed):
+                    out.append(PagedView({name: t[index] for name, t in g['tensors'].items()}, self.page_size, writes, group))
+                else:
+                    out.append(KVView(g['k'][index], g['v'][index], self.page_size, writes, group))
             else:
                 out.append(StateView(self.state_groups[group]['state'][index], writes, group))
         return out
 
     def bytes_per_token(self):
         size = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * len(g['entries']) * g['need'].kv_heads * g['need'].head_dim * size for g in self.kv_groups)
+        total = 0
+        for g in self.kv_groups:
+            need = g['need']
+            if isinstance(need, PagedNeed):
+                per_token = sum(_count(shape) * (4 if kind == 'float32' else size) for _, shape, kind in need.tensors)
+            else:
+                per_token = 2 * need.kv_heads * need.head_dim * size
+            total += len(g['entries']) * per_token
+        return total
+
+
+def _count(shape):
+    n = 1
+    for extent in shape:
+        n *= extent
+    return n

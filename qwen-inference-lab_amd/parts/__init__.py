@@ -1,5 +1,5 @@
 """Parts that models are assembled from."""
-from .base import (ParamSpec, KVNeed, StateNeed, Part, Norm, PositionEncoding, Rotation,
+from .base import (ParamSpec, KVNeed, PagedNeed, StateNeed, Part, Norm, PositionEncoding, Rotation,
                    Mixer, FeedForward, Block)
 from .norm import RMSNorm
 from .rotary import Rotary
@@ -9,6 +9,6 @@ from .block import PreNormBlock
 from .embedding import Embedding, LMHead
 from .model import CausalLM, ScheduleEntry
 
-__all__ = ['ParamSpec', 'KVNeed', 'StateNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
+__all__ = ['ParamSpec', 'KVNeed', 'PagedNeed', 'StateNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
            'FeedForward', 'Block', 'RMSNorm', 'Rotary', 'Attention', 'GatedMLP', 'PreNormBlock',
            'Embedding', 'LMHead', 'CausalLM', 'ScheduleEntry']

@@ -30,6 +30,17 @@ class KVNeed:
 
 
 @dataclass(frozen=True)
+class PagedNeed:
+    """Per-token data in pages, in tensors of the mixer's own: ``tensors`` is a tuple of (name, shape of one
+    token's entry, 'model' or 'float32').  The cache manager keeps ``[pages, page_size, *shape]`` per name and entry
+    and gives the mixer a ``PagedView`` with the step's block tables and the new tokens' slots (slot = page *
+    page_size + position % page_size, an index into the first two axes taken together).  ``window`` None keeps every
+    token; needs that are equal share a page pool and block tables."""
+    tensors: tuple
+    window: int | None = None
+
+
+@dataclass(frozen=True)
 class StateNeed:
     """Fixed-size per-request state, one slot per live request.
 

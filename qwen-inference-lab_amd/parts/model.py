@@ -3,7 +3,7 @@ from dataclasses import dataclass
 
 import torch
 
-from .base import KVNeed, StateNeed
+from .base import KVNeed, PagedNeed, StateNeed
 from .. import ops
 
 
@@ -69,11 +69,11 @@ class CausalLM:
         return out
 
     def cache_needs(self):
-        """Per schedule entry: KVNeed | StateNeed | None, or ('shared', owner position)."""
+        """Per schedule entry: KVNeed | PagedNeed | StateNeed | None, or ('shared', owner position)."""
         needs = []
         for entry in self.schedule:
             need = self._need(entry)
-            if need is not None and not isinstance(need, (KVNeed, StateNeed)):
+            if need is not None and not isinstance(need, (KVNeed, PagedNeed, StateNeed)):
                 raise TypeError(f'unknown cache need {need!r}')
             needs.append(need if entry.cache_of is None or need is None else ('shared', entry.cache_of))
         return needs

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from qil_amd.cache import CacheManager, CacheFull, PagePool
-from qil_amd.parts import KVNeed, StateNeed
+from qil_amd.parts import KVNeed, PagedNeed, StateNeed
 
 
 def manager(needs=None, pages=4, page_size=2, requests=4, **kwargs):
@@ -86,6 +86,34 @@ def test_groups_of_layers_with_different_needs():
     cache.release('r')
     cache.check()
     assert cache.free_pages == [6, 5]
+
+
+def test_paged_needs_of_a_mixers_own():
+    """A need of per-token tensors of a mixer's own gets a page group like keys and values: equal needs share pool and
+    tables, a window gives pages back, the storage is [entries, pages, page_size, *shape] per name."""
+    latent = PagedNeed((('latent', (5,), 'float32'), ('code', (2, 3), 'model')))
+    needs = [KVNeed(1, 8, None), latent, latent, PagedNeed((('latent', (5,), 'float32'),), window=3), ('shared', 1)]
+    cache = CacheManager(needs, num_pages=[4, 4, 6], page_size=2, max_requests=2, dtype=torch.bfloat16, device='cpu',
+                         max_step_tokens=2)
+    assert [g['entries'] for g in cache.kv_groups] == [[0], [1, 2], [3]]
+    tensors = cache.kv_groups[1]['tensors']
+    assert tensors['latent'].shape == (2, 4, 2, 5) and tensors['latent'].dtype == torch.float32
+    assert tensors['code'].shape == (2, 4, 2, 2, 3) and tensors['code'].dtype == torch.bfloat16
+    views = cache.views()
+    assert views[2].tensors['code'].shape == (4, 2, 2, 3) and views[2].writes and views[2].group == 1
+    assert not views[4].writes and views[4].tensors['latent'].data_ptr() == views[1].tensors['latent'].data_ptr()
+    assert cache.bytes_per_token() == 2 * 8 * 2 + 2 * (5 * 4 + 6 * 2) + 5 * 4
+    assert cache.admit('r', 8)
+    at = 0
+    for step in (2, 2, 2, 2):
+        cache.ensure('r', at + step)
+        at += step
+        cache.advance('r', at)
+        cache.check()
+    assert all(p >= 0 for p in cache.table(1, 'r')) and cache.table(2, 'r')[:2] == [-1, -1]
+    cache.release('r')
+    cache.check()
+    assert cache.free_pages == [4, 4, 6]
 
 
 def test_window_never_frees_a_visible_key():

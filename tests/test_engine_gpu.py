@@ -348,6 +348,137 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     assert not torch.allclose(last[0], whole['a'][-1], atol=1e-3)
 
 
+def test_toy_mixer_with_a_paged_cache_of_its_own(tmp_path):
+    """A mixer that keeps ONE latent vector a token in pages (no heads, no keys and values: a ``PagedNeed`` with a
+    tensor of its own) becomes an architecture without a change to the framework: a token's output is the mean of
+    the latents up to it, projected back.  Whole prompts, portions and mixed batches over so few pages that they are
+    used again agree with each other and with a float64 restatement; the pool is poisoned first."""
+    from qil_amd import ops
+    from qil_amd.engine import ModelRunner, StepEntry
+    from qil_amd.parts import (Mixer, ParamSpec, PagedNeed, RMSNorm, GatedMLP, PreNormBlock, Embedding, LMHead, CausalLM,
+                               ScheduleEntry)
+    from qil_amd.registry import register_architecture
+    from qil_amd.weights import write_random_model, load_model
+
+    latent = 24
+
+    class LatentMean(Mixer):
+        graph_safe = False                                            # it reads the host side of the step
+
+        def __init__(self, width, dtype):
+            super().__init__()
+            self.width, self.dtype = width, dtype
+
+        def param_specs(self):
+            return {'down.weight': ParamSpec((latent, self.width)), 'up.weight': ParamSpec((self.width, latent))}
+
+        def cache_need(self):
+            return PagedNeed((('latent', (latent,), 'float32'),))
+
+        def forward(self, h, ctx, cache):
+            z = ops.linear(h, self.p['down.weight'], None).float()
+            store = cache.tensors['latent'].view(-1, latent)          # [pages * page_size, latent]: a slot is a row
+            if cache.writes:
+                store[cache.slots.long()] = z
+            out = torch.empty_like(z)
+            for s in range(ctx.n_seqs):
+                a, b, start = ctx.host_cu_seqlens[s], ctx.host_cu_seqlens[s + 1], ctx.host_starts[s]
+                end = start + b - a
+                positions = torch.arange(end, device=h.device)
+                pages = cache.block_tables[s].long()[positions // cache.page_size]
+                history = store[pages * cache.page_size + positions % cache.page_size]       # the request's latents in order
+                sums = torch.cumsum(history, dim=0)[start:end]
+                out[a:b] = sums / torch.arange(start + 1, end + 1, device=h.device)[:, None]
+            return ops.linear(out.to(self.dtype), self.p['up.weight'], None)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        intermediate_size: int
+        num_hidden_layers: int
+        rms_norm_eps: float = 1e-6
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(**{k: data[k] for k in cls.__dataclass_fields__ if k in data})
+
+        def to_dict(self):
+            return dict(self.__dict__, architectures=['ToyLatentLM'], model_type='toy_latent')
+
+    def build(config, *, dtype, device):
+        embedding = Embedding(config.vocab_size, config.hidden_size)
+        blocks = [PreNormBlock(mixer_norm=RMSNorm(config.hidden_size, config.rms_norm_eps),
+                               mixer=LatentMean(config.hidden_size, dtype),
+                               ffn_norm=RMSNorm(config.hidden_size, config.rms_norm_eps),
+                               ffn=GatedMLP(width=config.hidden_size, intermediate=config.intermediate_size, dtype=dtype),
+                               dtype=dtype) for _ in range(config.num_hidden_layers)]
+        final_norm, head = RMSNorm(config.hidden_size, config.rms_norm_eps), LMHead(config.vocab_size, config.hidden_size)
+        names = {'embed.weight': (embedding, 'weight'), 'norm.weight': (final_norm, 'weight'), 'head.weight': (head, 'weight')}
+        for i, block in enumerate(blocks):
+            for prefix, part in block.parts().items():
+                for local in part.param_specs():
+                    names[f'layers.{i}.{prefix}.{local}'] = (part, local)
+        return CausalLM(config=config, embedding=embedding, blocks=blocks,
+                        schedule=[ScheduleEntry(i) for i in range(len(blocks))], final_norm=final_norm, head=head,
+                        names=names, dtype=dtype, device=device)
+
+    register_architecture('ToyLatentLM', model_type='toy_latent', config_class=ToyConfig, build=build, replace=True)
+    data = dict(architectures=['ToyLatentLM'], model_type='toy_latent', vocab_size=90, hidden_size=40, intermediate_size=64,
+                num_hidden_layers=2)
+    folder = write_random_model(tmp_path / 'toy', data, seed=9)
+    model = load_model(folder, dtype=torch.float32, device='cuda')
+    prompts = dict(zip('abc', prompts_for(data, [23, 9, 14], 7)))
+
+    def run(steps, pages):
+        """steps: lists of (request, tokens taken); a request is admitted at its first step and released at its last."""
+        runner = ModelRunner(model, num_pages=pages, page_size=4, max_requests=2)
+        group = runner.cache.kv_groups[0]
+        assert set(group['tensors']) == {'latent'} and group['tensors']['latent'].shape == (2, pages, 4, latent)
+        group['tensors']['latent'].fill_(float('nan'))
+        got, at = {r: [] for r in prompts}, {r: 0 for r in prompts}
+        for step in steps:
+            entries = []
+            for request, size in step:
+                if at[request] == 0:
+                    assert runner.admit(request)
+                entries.append(StepEntry(request, tuple(prompts[request][at[request]:at[request] + size]), tuple(range(size))))
+            logits = runner.step(entries)
+            row = 0
+            for entry in entries:
+                got[entry.request].append(logits[row:row + len(entry.tokens)])
+                row += len(entry.tokens)
+                at[entry.request] += len(entry.tokens)
+                if at[entry.request] == len(prompts[entry.request]):
+                    runner.release(entry.request)
+            runner.cache.check()
+        assert runner.cache.free_pages == [pages]
+        return {r: torch.cat(parts) for r, parts in got.items() if parts}
+
+    whole = run([[('a', 23)], [('b', 9)], [('c', 14)]], pages=6)
+    # a and b live together, then c takes b's place and pages: 6 + 4 pages at most, of 10
+    mixed = run([[('a', 5), ('b', 2)], [('b', 1), ('a', 9)], [('a', 1), ('b', 6)], [('c', 3), ('a', 4)], [('a', 4), ('c', 10)],
+                 [('c', 1)]], pages=10)
+    for r in prompts:
+        assert torch.isfinite(whole[r]).all()
+        torch.testing.assert_close(mixed[r], whole[r], atol=1e-5, rtol=1e-4)
+    # float64 restatement of the whole model for request a
+    from safetensors.torch import load_file
+    w = {k: v.double() for k, v in load_file(str(folder / 'model.safetensors')).items()}
+    def norm(x, g): return x * torch.rsqrt(x.square().mean(-1, keepdim=True) + 1e-6) * g
+    x = w['embed.weight'][torch.tensor(prompts['a'])]
+    for i in range(2):
+        z = norm(x, w[f'layers.{i}.mixer_norm.weight']) @ w[f'layers.{i}.mixer.down.weight'].t()
+        means = torch.cumsum(z, 0) / torch.arange(1, len(z) + 1)[:, None]
+        x = x + means @ w[f'layers.{i}.mixer.up.weight'].t()
+        y = norm(x, w[f'layers.{i}.ffn_norm.weight'])
+        gate, up = y @ w[f'layers.{i}.ffn.gate_proj.weight'].t(), y @ w[f'layers.{i}.ffn.up_proj.weight'].t()
+        x = x + (torch.nn.functional.silu(gate) * up) @ w[f'layers.{i}.ffn.down_proj.weight'].t()
+    expected = norm(x, w['norm.weight']) @ w['head.weight'].t()
+    torch.testing.assert_close(whole['a'].double().cpu(), expected, atol=2e-5, rtol=2e-4)
+
+
 def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
     """Parts the framework does not have, defined here and used without a change to its files: a feed-forward
     that routes each token to one of three experts (router logits in float32), and a position encoding that
