@@ -273,7 +273,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
                        int table_stride, const int* row_seq, const int* positions, const int* row_index,
                        float* part_acc, float* part_m,
                        float* part_l, void* out, int rows, int heads, int kv_heads, int d, int page_size, int window,
-                       float scale, int P, int parts, hipStream_t s) {
+                       float scale, int P, int parts, hipStream_t s, bool merge = true) {
   const int g = heads / kv_heads;
   const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;            // head tile: 1, 2, 4 or 8
   const int tg_log2 = next_pow2_log2((d + 7) / 8);
@@ -292,7 +292,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
   }
 #undef QIL_ROWS_CASE
   int status = (int)hipGetLastError();
-  if (status || parts == 1) return status;
+  if (status || parts == 1 || !merge) return status;
   int tg;
   dim3 merge_grid;
   merge_shape(rows, heads, d, &tg, &merge_grid);
@@ -331,6 +331,28 @@ int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* 
                               acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
   return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+}
+
+// The same without the merge: the parts' results stay in the workspace for a consumer that merges them itself
+// (parts > 1; `out` is not written).
+int qil_attn_rows_unmerged(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
+                           int table_stride, const int* row_seq, const int* positions, void* workspace, int rows,
+                           int heads, int kv_heads, int d, int page_size, int window, float scale, int P, int parts,
+                           int dtype, hipStream_t s) {
+  if (rows == 0) return 0;
+  if (d % 8 || d > 256 || d < 8 || heads % kv_heads || P < 1 || P > 1024 || parts < 2 || parts > 65535 ||
+      kv_heads > 65535 || !workspace) return -1;
+  const int g = heads / kv_heads;
+  const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;
+  if (rows_lds_floats(gt, P, d) * sizeof(float) > 64 * 1024) return -1;
+  float* acc = (float*)workspace;
+  float* m = acc + (size_t)rows * heads * parts * d;
+  float* l = m + (size_t)rows * heads * parts;
+  if (dtype == QIL_F32)
+    return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, nullptr,
+                              acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s, false);
+  return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, nullptr,
+                             acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s, false);
 }
 
 // Merge of partial results written by a partial kernel (this file's or the matrix-core decode kernel's).

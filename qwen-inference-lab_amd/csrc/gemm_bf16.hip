@@ -22,6 +22,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "merge_parts.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -162,71 +163,14 @@ static int launch_stream(const bf16_t* A, const bf16_t* W, const float* bias, OU
 // Takes M <= 16, K a multiple of 128 per split, 16-byte aligned operands, no bias.
 #define LINES_WAVES 8
 
-// A given as the unmerged partial results of split-context attention (attention_rows.hip,
-// attention_decode.hip): acc [M, heads, parts, d], m and l [M, heads, parts], float32.  Row m, column
-// head * d + e of A is sum_p acc_p[e] exp(m_p - max m) / sum_p l_p exp(m_p - max m) over the parts that
-// hold keys of the row: the merge of attn_rows_merge_kernel, made while A is staged.
-struct UnmergedA {
-  const float* acc;
-  const float* m;
-  const float* l;
-  const int* positions;                                    // [M]: a row's context is its position + 1
-  int heads, d, parts, P, window;
-};
 #define LINES_DEPTH 3                                      // stages of W in flight per wave
 #define LINES_LDS_LIMIT (100 * 1024)                       // one block of 8 waves on a CU when A is long, two otherwise
 
 // Eight merged values of row m starting at column k (all of one head: d % 8 == 0), as bfloat16.
 __device__ __forceinline__ uint4 merged8(const UnmergedA& u, int m, int k) {
-  const int head = k / u.d, e = k - head * u.d;
-  const int ctx = u.positions[m] + 1;
-  const int lo = u.window > 0 ? max(0, ctx - u.window) : 0;
-  const int first = lo / u.P, last = (ctx - 1) / u.P;
-  const size_t cell0 = ((size_t)m * u.heads + head) * u.parts;
-  // four parts at a time, all their loads first: a loop that waits for memory once per part would cost more
-  // than the merge kernel it replaces.  The first four parts' sums and values are asked for together with their
-  // maxima (they do not depend on the largest maximum, only their use does): one wait for up to four parts.
-  float mv[4], lv[4], part[4][8];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int p = min(first + j, last);
-    mv[j] = u.m[cell0 + p];
-    lv[j] = u.l[cell0 + p];
-    ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
-  }
-  float top = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) top = fmaxf(top, mv[j]);
-  for (int p0 = first + 4; p0 <= last; p0 += 4) {
-    float more[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) more[j] = u.m[cell0 + min(p0 + j, last)];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) top = fmaxf(top, more[j]);
-  }
-  float denom = 0.f, numer[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int p0 = first; p0 <= last; p0 += 4) {
-    if (p0 != first) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int p = min(p0 + j, last);
-        mv[j] = u.m[cell0 + p];
-        lv[j] = u.l[cell0 + p];
-        ld8(u.acc + (cell0 + p) * u.d + e, part[j]);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {                           // the order and the arithmetic of the merge kernel
-      if (p0 + j <= last) {
-        const float f = expf(mv[j] - top);
-        denom += lv[j] * f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) numer[i] += part[j][i] * f;
-      }
-    }
-  }
-  return make_uint4(pack_bf16(numer[0] / denom, numer[1] / denom), pack_bf16(numer[2] / denom, numer[3] / denom),
-                    pack_bf16(numer[4] / denom, numer[5] / denom), pack_bf16(numer[6] / denom, numer[7] / denom));
+  float v[8];
+  merged_values<8>(u, m, k, v);
+  return make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
 }
 
 // A given as the float32 residual stream whose RMSNorm is to be taken (qil/model.py:15-23), with the rows' sums of

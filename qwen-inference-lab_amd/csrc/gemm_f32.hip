@@ -9,6 +9,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "merge_parts.h"
 
 #define SG_BM 64
 #define SG_BN 64
@@ -195,9 +196,19 @@ gemm_f32_stream_kernel(const float* __restrict__ A, const float* __restrict__ W,
 #define FL_DEPTH 3                                         // stages of W in flight per wave
 #define FL_LDS_LIMIT (100 * 1024)
 
+// A given as the gate and up products of a gated feed-forward, left as partial sums: sums [splits][M][2 K] with
+// the gate columns first or (interleaved) gate and up columns in turns of 16.  Row m, column k of A is
+// silu(gate[m, k]) * up[m, k] with both summed in split order: what silu_mul in elementwise.hip makes (qil/model.py:71).
+struct GatedA {
+  const float* sums;
+  int splits, interleaved;
+};
+
+// ASRC: 0 = A as it is, 1 = merged attention parts (UnmergedA), 2 = the activation of a gated feed-forward (GatedA)
+template <int ASRC>
 __global__ void __launch_bounds__(FL_WAVES * QIL_WAVE)
-gemm_f32_lines_kernel(const float* __restrict__ A, const float* __restrict__ W, float* __restrict__ C, int M, int N,
-                      int K, int cols_per_split) {
+gemm_f32_lines_kernel(const float* __restrict__ A, UnmergedA unmerged, GatedA gated, const float* __restrict__ W,
+                      float* __restrict__ C, int M, int N, int K, int cols_per_split) {
   extern __shared__ __align__(16) float fl_lds[];           // A slice [8 or 16][cols + pad], then the waves' buffers
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
@@ -221,7 +232,37 @@ gemm_f32_lines_kernel(const float* __restrict__ A, const float* __restrict__ W, 
   for (int idx = threadIdx.x; idx < a_rows * (cols_per_split / 4); idx += FL_WAVES * QIL_WAVE) {
     const int m = idx / (cols_per_split / 4), c = (idx - m * (cols_per_split / 4)) * 4;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (m < M) v = *reinterpret_cast<const float4*>(A + (size_t)m * K + k_begin + c);
+    if (m < M) {
+      if (ASRC == 1) {
+        float merged[4];
+        merged_values<4, 16>(unmerged, m, k_begin + c, merged);
+        v = make_float4(merged[0], merged[1], merged[2], merged[3]);
+      } else if (ASRC == 2) {
+        const int k = k_begin + c;                          // four columns of one tile of 16
+        const size_t at = (size_t)m * 2 * K + (gated.interleaved ? (size_t)(k >> 4) * 32 + (k & 15) : (size_t)k);
+        const size_t stride = (size_t)M * 2 * K;
+        float4 g = make_float4(0.f, 0.f, 0.f, 0.f), u = g;
+        for (int s0 = 0; s0 < gated.splits; s0 += 4) {       // four splits' loads at a time; the sums in split order
+          float4 gs[4], us[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const size_t from = (size_t)min(s0 + j, gated.splits - 1) * stride + at;
+            gs[j] = *reinterpret_cast<const float4*>(gated.sums + from);
+            us[j] = *reinterpret_cast<const float4*>(gated.sums + from + (gated.interleaved ? 16 : K));
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (s0 + j < gated.splits) {
+              g.x += gs[j].x; g.y += gs[j].y; g.z += gs[j].z; g.w += gs[j].w;
+              u.x += us[j].x; u.y += us[j].y; u.z += us[j].z; u.w += us[j].w;
+            }
+        }
+        v = make_float4((g.x / (1.f + expf(-g.x))) * u.x, (g.y / (1.f + expf(-g.y))) * u.y,
+                        (g.z / (1.f + expf(-g.z))) * u.z, (g.w / (1.f + expf(-g.w))) * u.w);
+      } else {
+        v = *reinterpret_cast<const float4*>(A + (size_t)m * K + k_begin + c);
+      }
+    }
     *reinterpret_cast<float4*>(a_lds + m * row_width + c) = v;
   }
   // every wave walks its K range from a start of its own and wraps around (waves that read the same columns
@@ -306,6 +347,60 @@ static int fl_splits(int M, int N, int K) {
   return fit;
 }
 
+template <int ASRC>
+static int launch_f32_lines(const float* A, UnmergedA unmerged, GatedA gated, const float* W, float* C, int M, int N, int K,
+                            int splits, hipStream_t s) {
+  const size_t lds = fl_lds_bytes(M, K, splits);
+  auto kernel = gemm_f32_lines_kernel<ASRC>;
+  static size_t granted = 0;                              // per instantiation
+  if (lds > 64 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((N + 16 * FL_WAVES - 1) / (16 * FL_WAVES), 1, splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(FL_WAVES * QIL_WAVE), lds, s, A, unmerged, gated, W, C, M, N, K, K / splits);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// The whole-line product with the merge of split-context attention results made while A is staged
+// (A[M, heads * d] is never written).  workspace: acc [M, heads, parts, d], then m and l [M, heads, parts], float32
+// (attention_rows.hip).  C float32 [splits, M, N].
+extern "C" int qil_gemm_f32_unmerged_takes(int M, int N, int heads, int d, int splits) {
+  return heads >= 1 && d >= 4 && d % 4 == 0 && splits >= 1 && fl_takes(M, N, heads * d, splits);
+}
+
+extern "C" int qil_gemm_f32_unmerged(const void* workspace, const int* positions, const void* W, float* C, int M, int N,
+                                     int heads, int d, int window, int P, int parts, int splits, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  if (!qil_gemm_f32_unmerged_takes(M, N, heads, d, splits) || parts < 1 || P < 1 ||
+      (((uintptr_t)workspace | (uintptr_t)W) % 16))
+    return -1;
+  UnmergedA u;
+  u.acc = (const float*)workspace;
+  u.m = u.acc + (size_t)M * heads * parts * d;
+  u.l = u.m + (size_t)M * heads * parts;
+  u.positions = positions;
+  u.heads = heads; u.d = d; u.parts = parts; u.P = P; u.window = window;
+  return launch_f32_lines<1>(nullptr, u, GatedA(), (const float*)W, C, M, N, heads * d, splits, s);
+}
+
+// The whole-line product of the activation of a gated feed-forward, made from the gate and up products' partial
+// sums while A is staged: sums float32 [sum_splits, M, 2 K].  C float32 [splits, M, N].
+extern "C" int qil_gemm_f32_gated_takes(int M, int N, int K, int interleaved, int splits) {
+  return splits >= 1 && (!interleaved || K % 16 == 0) && fl_takes(M, N, K, splits);
+}
+
+extern "C" int qil_gemm_f32_gated(const float* sums, int sum_splits, int interleaved, const void* W, float* C, int M, int N,
+                                  int K, int splits, hipStream_t s) {
+  if (M == 0 || N == 0) return 0;
+  if (!qil_gemm_f32_gated_takes(M, N, K, interleaved, splits) || sum_splits < 1 || (((uintptr_t)sums | (uintptr_t)W) % 16))
+    return -1;
+  GatedA g;
+  g.sums = sums; g.splits = sum_splits; g.interleaved = interleaved;
+  return launch_f32_lines<2>(nullptr, UnmergedA(), g, (const float*)W, C, M, N, K, splits, s);
+}
+
 extern "C" int qil_gemm_f32_mfma_takes(int M, int N, int K, int splits);      // gemm_f32_mfma.hip
 extern "C" long qil_gemm_f32_mfma_blocks(int M, int N);
 extern "C" int qil_gemm_f32_mfma_splits(int M, int N, int K);
@@ -351,18 +446,8 @@ extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, f
       (((uintptr_t)A | (uintptr_t)W | (uintptr_t)C) % 16) == 0)
     return qil_gemm_f32_mfma(A, W, bias, C, M, N, K, splits, s);
   if (splits > 1 && (!stream_ok || bias)) return -1;
-  if (stream_ok && !bias && splits == fl_splits(M, N, K) && fl_takes(M, N, K, splits)) {
-    const size_t lds = fl_lds_bytes(M, K, splits);
-    static size_t granted = 0;
-    if (lds > 64 * 1024 && lds > granted) {
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_f32_lines_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return (int)e;
-      granted = lds;
-    }
-    dim3 grid((N + 16 * FL_WAVES - 1) / (16 * FL_WAVES), 1, splits);
-    hipLaunchKernelGGL(gemm_f32_lines_kernel, grid, dim3(FL_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
-    QIL_RETURN_LAUNCH_STATUS();
-  }
+  if (stream_ok && !bias && (splits == 1 || splits == fl_splits(M, N, K)) && fl_takes(M, N, K, splits))
+    return launch_f32_lines<0>(A, UnmergedA(), GatedA(), W, C, M, N, K, splits, s);
   if (stream_ok) {
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;           // 16-row tiles of A a block keeps
     const int steps = (K + 15) / 16, steps_per_split = (steps + splits - 1) / splits;

@@ -46,6 +46,8 @@ DECODE_MAX_PART = 8192
 # launch (64 rows of 2048 keys: 111 us against 94 + 5; whole steps at 8B sizes: 24 and 32 rows gain 0.8 %
 # with the fused kernel, 48 rows lose 2 %).
 FUSED_DECODE_MOST_ROWS = 32
+# Rows up to which the row kernel leaves its parts unmerged when the caller allows (the product after it merges them).
+UNMERGED_ROWS_MOST = 16
 # Launches of at most this many blocks (one a CU) let a wave load two of its steps at a time.
 DECODE_PAIRS_BLOCKS = 256
 
@@ -56,6 +58,15 @@ DECODE_PAIRS_BLOCKS = 256
 # steps, the pair wins with 9 to 16 rows (8B sizes: 12 rows 4.73 -> 4.66 ms, 16 rows 5.08 -> 4.91) and for small
 # products, which are bound by the number of kernels (0.6B sizes: 1 row 1.28 -> 1.23 ms, 8 rows 1.56 -> 1.54), and
 # is level with up to 8 rows of large ones (8B sizes, 8 rows: 4.27 -> 4.27), where it stays off.
+# A float32 product of up to 16 rows (the whole-line kernel's) may make its operand itself while it stages it: the
+# merge of the attention's context parts (``Unmerged``) or the activation of the gated feed-forward before it
+# (``Gated``).  That saves a kernel, and every block of 128 result columns repeats the work for its slice of K: it pays
+# while rows x K x blocks of columns is small.  Measured on whole float32 decode steps (merge / activation alone):
+# 0.6B sizes 4 rows -2.4 % / -2.3 %, 16 rows +0.4 / -0.7; 8B sizes 1 row -0.9 / -1.0, 4 rows -0.6 / -0.8, 8 rows
+# +1.6 / +1.6; 32B sizes 1 row -1.2 / -1.9, 2 rows +2.0 / +0.4, 4 rows +4.2 / +0.1.
+GATED_OPERAND_MOST_ROWS = 16
+UNMERGED_OPERAND_MOST_WORK = 1 << 19
+GATED_OPERAND_MOST_WORK = 1 << 21
 NORMED_GEMM_MOST_ROWS = 16
 ADD_GEMM_MOST_ROWS = 16
 ADD_GEMM_FEW_ROWS = 8                 # up to this many rows only products of at most ...
@@ -93,6 +104,21 @@ class Unmerged:
                                              self.shape[0], self.heads, self.head_dim, self.window, self.part,
                                              self.parts, _code(self.dtype), _stream()), 'attn_merge')
         return self.out
+
+
+class Gated:
+    """The activation of a gated feed-forward, silu(gate) * up, not computed yet: ``sums`` are the gate and up
+    products' partial sums (``Partials`` [N, 2 I]).  ``linear`` makes the activation while it stages its operand
+    when its kernel takes the sizes, which saves the activation kernel; ``materialize()`` runs that kernel."""
+
+    is_cuda = True
+
+    def __init__(self, sums, interleaved, dtype):
+        self.sums, self.interleaved, self.dtype = sums, bool(interleaved), dtype
+        self.shape, self.device = (sums.shape[0], sums.shape[1] // 2), sums.device
+
+    def materialize(self):
+        return silu_mul(self.sums, self.dtype, interleaved=self.interleaved)
 
 
 class Added:
@@ -235,6 +261,22 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False, add_to=None):
     ``x`` may be ``Unmerged`` attention results, or a ``Normed`` residual stream.
     ``add_to``: the float32 residual stream [N, O]; if the kernel for these sizes can add its result into it
     (every element complete before it is added), it does and an ``Added`` is returned instead of the result."""
+    if isinstance(x, Gated):
+        lib = library.load()
+        n, k = x.shape
+        o = weight.shape[0]
+        splits = lib.qil_gemm_f32_splits(n, o, k)
+        if partials and bias is None and out_dtype in (None, torch.float32) and x.dtype == torch.float32 and \
+                weight.dtype == torch.float32 and n <= GATED_OPERAND_MOST_ROWS and \
+                n * k * -(-o // 128) <= GATED_OPERAND_MOST_WORK and \
+                lib.qil_gemm_f32_gated_takes(n, o, k, int(x.interleaved), splits):
+            _require(x.sums.tensor, 'gate and up sums', torch.float32, (x.sums.splits, n, 2 * k))
+            _require(weight, 'weight', torch.float32, (o, k))
+            out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+            _check(lib.qil_gemm_f32_gated(_ptr(x.sums.tensor), x.sums.splits, int(x.interleaved), _ptr(weight), _ptr(out),
+                                          n, o, k, splits, _stream()), 'gemm_f32_gated')
+            return Partials(out)
+        x = x.materialize()
     if isinstance(x, Normed):
         lib = library.load()
         n, k = x.shape
@@ -277,6 +319,15 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False, add_to=None):
                                               x.heads, x.head_dim, x.window, x.part, x.parts, splits, _stream()),
                    'gemm_bf16_unmerged')
             return Partials(out)
+        if partials and bias is None and out_dtype in (None, x.dtype) and x.dtype == torch.float32:
+            splits = lib.qil_gemm_f32_splits(n, o, k)
+            if n * k * -(-o // 128) <= UNMERGED_OPERAND_MOST_WORK and \
+                    lib.qil_gemm_f32_unmerged_takes(n, o, x.heads, x.head_dim, splits):
+                out = torch.empty((splits, n, o), dtype=torch.float32, device=x.device)
+                _check(lib.qil_gemm_f32_unmerged(_ptr(x.workspace), _ptr(x.positions), _ptr(weight), _ptr(out), n, o,
+                                                 x.heads, x.head_dim, x.window, x.part, x.parts, splits, _stream()),
+                       'gemm_f32_unmerged')
+                return Partials(out)
         x = x.merge()
     _require(x, 'x')
     _require(weight, 'weight', x.dtype)
@@ -331,12 +382,13 @@ def interleave_gate_up(gate, up):
     return torch.stack((gate.view(inner // 16, 16, k), up.view(inner // 16, 16, k)), dim=1).reshape(2 * inner, k).contiguous()
 
 
-def gated_linear(x, weight, out_dtype=None, interleaved=False):
+def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False):
     """silu(x @ gate^T) * (x @ up^T) -> [N, I], with ``weight`` the [2 I, K] matrix of both: the gate rows stacked
     before the up rows, or (``interleaved``) both in turns of 16 rows, which the kernels read faster.
 
     One kernel when a fused kernel takes the sizes (bfloat16; up to 16 rows, or up to 256 rows of an interleaved
-    matrix large enough to fill the chip); otherwise the product followed by ``silu_mul``.  Both add in float32."""
+    matrix large enough to fill the chip); otherwise the product followed by ``silu_mul``.  Both add in float32.
+    ``lazy``: a few float32 rows may come back as ``Gated`` (the product's partial sums) for ``linear`` to finish."""
     if isinstance(x, Normed):
         x = x.materialize()
     _require(x, 'x')
@@ -361,7 +413,10 @@ def gated_linear(x, weight, out_dtype=None, interleaved=False):
         _check(lib.qil_gemm_bf16_gated(_ptr(x), _ptr(weight), _ptr(out), n, both // 2, k, _code(out_dtype), 0, 0,
                                        int(interleaved), _stream()), 'gemm_bf16_gated')
         return out
-    return silu_mul(linear(x, weight, None, partials=True), out_dtype, interleaved=interleaved)
+    sums = linear(x, weight, None, partials=True)
+    if lazy and x.dtype == torch.float32 and out_dtype == torch.float32 and n <= GATED_OPERAND_MOST_ROWS:
+        return Gated(sums if isinstance(sums, Partials) else Partials(sums[None]), interleaved, out_dtype)
+    return silu_mul(sums, out_dtype, interleaved=interleaved)
 
 
 def silu_mul(gate_up, out_dtype=None, interleaved=False):
@@ -592,6 +647,14 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             parts = max(1, -(-max_context // part))
             nbytes = lib.qil_attn_rows_workspace(rows, heads, head_dim, parts)
             workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=qkv.device) if nbytes else None
+            if unmerged and parts > 1 and single_rows is None and rows <= UNMERGED_ROWS_MOST:
+                _check(lib.qil_attn_rows_unmerged(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                                                  _ptr(block_tables), block_tables.shape[1], _ptr(row_seq),
+                                                  _ptr(positions), _ptr(workspace), rows, heads, kv_heads, head_dim,
+                                                  page_size, window_arg, float(scale), part, parts, _code(qkv.dtype),
+                                                  _stream()), 'attn_rows_unmerged')
+                return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
+                                part=part, parts=parts)
             _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                      block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                      _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,

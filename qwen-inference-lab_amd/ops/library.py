@@ -155,6 +155,16 @@ def _declare(lib):
     lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_splits.argtypes = [i, i, i]
+    lib.qil_gemm_f32_unmerged_takes.argtypes = [i, i, i, i, i]
+    lib.qil_gemm_f32_unmerged_takes.restype = i
+    lib.qil_gemm_f32_unmerged.argtypes = [p, p, p, p, i, i, i, i, i, i, i, i, p]
+    lib.qil_gemm_f32_unmerged.restype = i
+    lib.qil_gemm_f32_gated_takes.argtypes = [i, i, i, i, i]
+    lib.qil_gemm_f32_gated_takes.restype = i
+    lib.qil_gemm_f32_gated.argtypes = [p, i, i, p, p, i, i, i, i, p]
+    lib.qil_gemm_f32_gated.restype = i
+    lib.qil_attn_rows_unmerged.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_rows_unmerged.restype = i
     lib.qil_gemm_f32_mfma.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_mfma_takes.argtypes = [i, i, i, i]
     lib.qil_gemm_f32_mfma_splits.argtypes = [i, i, i]

@@ -32,7 +32,7 @@ class GatedMLP(FeedForward):
     adds_to_stream = True
 
     def forward(self, h, add_to=None):
-        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype, interleaved=self.interleaved)
+        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype, interleaved=self.interleaved, lazy=True)
         if add_to is not None and hidden.is_cuda:              # few rows: the down product adds into the stream itself
             return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True, add_to=add_to)
         return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

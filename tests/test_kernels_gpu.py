@@ -648,6 +648,79 @@ def test_linear_merges_unmerged_attention(ops, lengths, window, d, heads, kv_hea
     check(biased, merged.double() @ w.double().t() + rand(out_features, seed=5).double(), dtype, scale=2)
 
 
+@pytest.mark.parametrize('lengths,window,d,heads,kv_heads,out_features,page_size', [
+    ([2100, 1, 700, 1290, 64, 2047, 300, 1500], None, 128, 16, 8, 1024, 16),      # Qwen3-0.6B sizes, 8 rows
+    ([900, 2100, 33], 500, 128, 32, 4, 300, 16),                                # a window; columns that fill no block
+    ([700], None, 64, 5, 5, 77, 8),                                            # one row, one head a kv head
+    ([3000, 5, 1200, 64, 65, 800, 90, 2300, 400, 17, 1000, 2000, 1, 300, 600, 1900], None, 40, 8, 2, 200, 16),   # 16 rows, d = 40
+    ([600, 700], None, 40, 3, 1, 50, 4),                                       # K no whole stage: merged first
+    ([600] * 17, None, 64, 4, 2, 64, 16),                                      # 17 rows: merged by the attention
+])
+def test_linear_float32_merges_unmerged_attention(ops, lengths, window, d, heads, kv_heads, out_features, page_size):
+    """The float32 output projection of up to 16 rows merges the row kernel's context parts while it stages its
+    operand: bit for bit what the merge kernel followed by the product gives."""
+    dtype = torch.float32
+    k_cache, v_cache, table, _ = build_cache(lengths, page_size, kv_heads, d, dtype)
+    rows = len(lengths)
+    q = rand(rows, heads * d, dtype=dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
+                block_tables=table, row_seq=torch.arange(rows, dtype=torch.int32).cuda(), positions=positions,
+                cu_seqlens=None, seq_starts=None, single_rows=None, n_seqs=rows, max_query=1, max_context=max(lengths),
+                scale=d ** -0.5, window=window)
+    w = rand(out_features, heads * d, dtype=dtype, seed=3, scale=(heads * d) ** -0.5)
+    merged = ops.paged_attention(q, **args)
+    assert isinstance(merged, torch.Tensor)
+    want = ops.linear(merged, w, None, partials=True)
+    lazy = ops.paged_attention(q, unmerged=True, **args)
+    if rows > 16:
+        assert isinstance(lazy, torch.Tensor)
+        torch.testing.assert_close(lazy, merged, atol=0, rtol=0)
+        return
+    assert isinstance(lazy, ops.Unmerged), 'several context parts and only single rows: nothing to merge yet'
+    got = ops.linear(lazy, w, None, partials=True)
+    fused = bool(ops.library.load().qil_gemm_f32_unmerged_takes(rows, out_features, heads, d, got.splits if isinstance(got, ops.Partials) else 1))
+    assert fused == ((heads * d) % 64 == 0 and heads * d >= 192)
+    as_tensor = lambda r: r.tensor if isinstance(r, ops.Partials) else r[None]
+    torch.testing.assert_close(as_tensor(got), as_tensor(want), atol=0, rtol=0)
+    torch.testing.assert_close(lazy.merge(), merged, atol=0, rtol=0)
+    check(as_tensor(got).sum(0), merged.double() @ w.double().t(), dtype, scale=2)
+    biased = ops.linear(ops.paged_attention(q, unmerged=True, **args), w, rand(out_features, seed=5))     # no fused path: merges first
+    check(biased, merged.double() @ w.double().t() + rand(out_features, seed=5).double(), dtype, scale=2)
+
+
+@pytest.mark.parametrize('rows,width,inner,interleaved', [
+    (1, 1024, 3072, True), (8, 1024, 3072, True), (16, 320, 192, True), (5, 200, 256, False), (3, 64, 448, True),
+    (2, 48, 100, False),                                      # K no whole stage: the activation kernel runs
+    (17, 128, 256, True),                                     # too many rows: the activation kernel runs
+])
+def test_linear_float32_makes_the_gated_activation(ops, rows, width, inner, interleaved):
+    """A float32 down product of up to 16 rows takes the gate and up products' partial sums and makes silu(gate) * up
+    while it stages its operand: bit for bit what the activation kernel followed by the product gives."""
+    x = rand(rows, width)
+    gate, up = rand(inner, width, seed=1, scale=width ** -0.5), rand(inner, width, seed=2, scale=width ** -0.5)
+    both = ops.interleave_gate_up(gate, up) if interleaved else torch.cat([gate, up]).contiguous()
+    down = rand(width + 8, inner, seed=3, scale=inner ** -0.5)
+    hidden = ops.gated_linear(x, both, torch.float32, interleaved=interleaved)
+    assert isinstance(hidden, torch.Tensor)
+    check(hidden, torch.nn.functional.silu(x.double() @ gate.double().t()) * (x.double() @ up.double().t()), torch.float32, scale=2)
+    want = ops.linear(hidden, down, None, partials=True)
+    lazy = ops.gated_linear(x, both, torch.float32, interleaved=interleaved, lazy=True)
+    if rows > 16:
+        assert isinstance(lazy, torch.Tensor)
+        torch.testing.assert_close(lazy, hidden, atol=0, rtol=0)
+        return
+    assert isinstance(lazy, ops.Gated)
+    torch.testing.assert_close(lazy.materialize(), hidden, atol=0, rtol=0)
+    got = ops.linear(lazy, down, None, partials=True)
+    as_tensor = lambda r: r.tensor if isinstance(r, ops.Partials) else r[None]
+    torch.testing.assert_close(as_tensor(got), as_tensor(want), atol=0, rtol=0)
+    check(as_tensor(got).sum(0), hidden.double() @ down.double().t(), torch.float32, scale=2)
+    whole = ops.linear(ops.gated_linear(x, both, torch.float32, interleaved=interleaved, lazy=True), down)   # a tensor is asked for
+    assert isinstance(whole, torch.Tensor)
+    check(whole, hidden.double() @ down.double().t(), torch.float32, scale=2)
+
+
 @pytest.mark.parametrize('lengths,page_size,d,heads,kv_heads,window,norm,rot,splits', [
     ([2100, 1, 700, 1290, 64, 2047, 300, 33], 16, 128, 32, 8, None, True, 128, 8),     # the benchmark's sizes
     ([1, 2, 31, 32, 33, 64, 65, 96], 8, 64, 6, 2, None, True, 64, 3),                  # every edge of a 32-key step and of a page
