@@ -55,7 +55,7 @@ def _halves(gate_up, interleaved):
     return tiles[:, :, 0].reshape(-1, inner), tiles[:, :, 1].reshape(-1, inner)
 
 
-def gated_linear(x, weight, out_dtype=None, interleaved=False):
+def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False):
     y = x.to(torch.float32) @ weight.to(torch.float32).t()
     g, u = _halves(y, interleaved)
     return (g / (1 + torch.exp(-g)) * u).to(out_dtype or x.dtype)
