@@ -172,7 +172,7 @@ def main():
         # One request's prompt arrives in portions while `batch` others decode: every step is one batch of
         # portion + batch rows, the decoding requests at --history tokens, the prompt growing from --history on.
         steps = min(args.steps, 12)
-        room = args.history + steps * args.portion + 16
+        room = args.history + (steps + 1) * args.portion + 16
         config_room = config['max_position_embeddings']
         if room > config_room:
             raise SystemExit(f'--history {args.history} and {steps} portions of {args.portion} need {room} positions, the model has {config_room}')

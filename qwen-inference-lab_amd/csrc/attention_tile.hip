@@ -21,6 +21,8 @@
 //   O^T[dim, row] = sum_key V^T[dim, key] P^T[key, row]    A = V tile transposed in LDS
 // bfloat16 uses v_mfma_f32_16x16x32_bf16 (P rounded to bfloat16, float32 accumulation); float32
 // uses v_mfma_f32_16x16x4_f32: float32 inputs and products, no reduced-precision mode.
+#include <algorithm>
+
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -60,7 +62,8 @@ __global__ void __launch_bounds__(TILE_THREADS, (sizeof(T) == 4 && DMAX > 64 && 
 attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                  const int* __restrict__ block_tables, int table_stride, const int* __restrict__ cu_seqlens,
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
-                 int page_size, int window, float scale, int GH, int chunks, int ps_shift) {
+                 int page_size, int window, float scale, int GH, int chunks, int ps_shift,
+                 float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P, int parts) {
   using TT = TileTraits<T>;
   constexpr int BK = TT::BK, KSTEP = TT::KSTEP, PAD = TT::PAD;
   constexpr bool BF16 = sizeof(T) == 2;
@@ -81,7 +84,12 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
   const int across = ((linear >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
   const int tile_row0 = across * block_rows;
   if (tile_row0 >= n) return;
-  const int kvh = blockIdx.z / chunks, chunk = blockIdx.z % chunks;
+  // parts > 1 (a few row tiles against a long context): grid.z also counts the parts of P keys, and a block
+  // leaves float32 partial results (the layout of the split-context row kernels) for the merge kernel
+  int pair = blockIdx.z;
+  const int part = pair / (kv_heads * chunks);
+  pair -= part * (kv_heads * chunks);
+  const int kvh = pair / chunks, chunk = pair % chunks;
   const int g = heads / kv_heads;
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   const int r = lane & 15, kb = lane >> 4;
@@ -93,8 +101,13 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
 
   const int rows_in_block = min(block_rows, n - tile_row0);
   const int pos_first = start + tile_row0;
-  const int key_end = pos_first + rows_in_block;                       // last position + 1
-  const int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  int key_end = pos_first + rows_in_block;                             // last position + 1
+  int key_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
+  if (parts > 1) {                                                     // P is a multiple of the tile's keys
+    key_begin = max(key_begin, part * P);
+    key_end = min(key_end, (part + 1) * P);
+    if (key_begin >= key_end) return;                                  // no row of the block sees a key of this part
+  }
 
   const int dt = WHOLE ? DMAX / 16 : (d + 15) / 16;    // dim tiles in use
   const int k_row = (BF16 ? (d + 31) / 32 * 32 : dt * 16) + PAD;       // elements per K row in LDS (staging
@@ -428,14 +441,29 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
     total += __shfl_xor(total, 16, QIL_WAVE);
     total += __shfl_xor(total, 32, QIL_WAVE);
     if (!row_valid[b]) continue;
-    const float inv = 1.f / total;
+    if (parts > 1) {
+      // acc [row, head, part, d] unnormalised, m (the maximum in the exponent's units) and l [row, head, part]; a row
+      // that sees no key of this part leaves m = -inf, l = 0 in a cell the merge does not read
+      const size_t cell = ((size_t)(q0 + my_row[b]) * heads + head) * parts + part;
+#pragma unroll
+      for (int t = 0; t < DTILES; ++t)
+        if (WHOLE || t * 16 + 4 * kb < d)                   // d % 4 == 0: the four dims are inside together
+          *reinterpret_cast<float4*>(part_acc + cell * d + t * 16 + 4 * kb) =
+              make_float4(o[b][t][0], o[b][t][1], o[b][t][2], o[b][t][3]);
+      if (kb == 0) {
+        part_m[cell] = m[b] == -INFINITY ? -INFINITY : m[b] * scale;
+        part_l[cell] = total;
+      }
+      continue;
+    }
+    // a division, as in the merge of parts: keys that all lie in one part then give the same bits either way
     T* orow = out + ((size_t)(q0 + my_row[b]) * heads + head) * d;
 #pragma unroll
     for (int t = 0; t < DTILES; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int dim = t * 16 + 4 * kb + i;
-        if (WHOLE || dim < d) st(orow + dim, o[b][t][i] * inv);
+        if (WHOLE || dim < d) st(orow + dim, o[b][t][i] / total);
       }
   }
 }
@@ -444,7 +472,7 @@ template <typename T, int DMAX, int RB>
 static int launch_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                        int max_query, int heads, int kv_heads, int d, int page_size, int window, float scale,
-                       hipStream_t s) {
+                       hipStream_t s, float* workspace = nullptr, int total_rows = 0, int P = 0, int parts = 1) {
   using TT = TileTraits<T>;
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
@@ -459,13 +487,16 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
     if (e != hipSuccess) return (int)e;
     granted[whole] = lds;
   }
-  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks);
+  if ((long)kv_heads * chunks * parts > 65535) return -1;
+  dim3 grid((max_query + 16 * RB * RT - 1) / (16 * RB * RT), n_seqs, kv_heads * chunks * parts);
+  float* part_m = workspace ? workspace + (size_t)total_rows * heads * parts * d : nullptr;
+  float* part_l = part_m ? part_m + (size_t)total_rows * heads * parts : nullptr;
   int ps_shift = -1;                                      // log2 of a power-of-two page size
   for (int b = 0; b < 30; ++b)
     if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(TILE_THREADS), lds, s, (const T*)q, q_stride, (const T*)k_cache,
                      (const T*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (T*)out, heads, kv_heads, d,
-                     page_size, window, scale, GH, chunks, ps_shift);
+                     page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts);
   return (int)hipGetLastError();
 }
 
@@ -476,20 +507,45 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
                                   const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
                                   int d, int page_size, int window, float scale, hipStream_t s);
 
+// Keys in parts for this file's kernel (the float32 path, and bfloat16 sizes that the branch-free kernel does not
+// take): a portion of a prompt deep in a long context is a few row tiles, each with all its keys ahead of it one
+// after the other, on fewer blocks than the chip has CUs.  Returns the number of parts to cut the keys into (1: do
+// not) and their size in *P: about two blocks a CU, parts of at least 128 keys, at most 32 of them.
+extern "C" int qil_attn_tile_key_parts(int n_seqs, int max_query, int heads, int kv_heads, int d, int max_context,
+                                       int dtype, int* P) {
+  *P = 0;
+  if (heads % kv_heads || max_query < 2 || max_context < 512) return 1;
+  const int g = heads / kv_heads, GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
+  const int RB = (dtype == QIL_BF16 && d <= 128) ? 2 : 1;
+  const long blocks = (long)((max_query + 16 * RB * RT - 1) / (16 * RB * RT)) * n_seqs * kv_heads * chunks;
+  if (blocks >= 256) return 1;
+  const int want = (int)std::min(32L, (512 + blocks - 1) / blocks);
+  int part = ((max_context + want - 1) / want + 63) / 64 * 64;         // whole tiles of 32 (float32) or 64 keys
+  part = std::max(part, 128);
+  const int parts = (max_context + part - 1) / part;
+  if (parts < 2 || (long)kv_heads * chunks * parts > 65535) return 1;
+  *P = part;
+  return parts;
+}
+
 // Sequences with >= 2 rows.  q: rows of stride q_stride, head h at h * d; out [rows, heads * d].
 // Requires d % 8 == 0, 8 <= d <= 256.  Returns -1 on a size it does not take.
-extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache,
-                             const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
-                             void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
-                             int window, float scale, int dtype, hipStream_t s) {
+// parts > 1: the keys in `parts` parts of P keys (P a multiple of 64) on this file's kernel; every row of a sequence
+// of two or more rows gets float32 partial results in `workspace` (qil_attn_rows_workspace bytes for all `total_rows`
+// rows of the step, indexed by the step's row) for qil_attn_merge, and `out` is not written.
+static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                         const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
+                         void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
+                         int window, float scale, int dtype, hipStream_t s, float* workspace, int total_rows, int P,
+                         int parts) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
-  if (dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
+  if (parts == 1 && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
     return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);
 #define QIL_TILE_CASE(T, DMAX)                                                                                      \
   return launch_tile<T, DMAX, (sizeof(T) == 2 && DMAX <= 128) ? 2 : 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
-                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s)
+                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s, workspace, total_rows, P, parts)
   if (dtype == QIL_F32) {
     if (d <= 64) QIL_TILE_CASE(float, 64);
     if (d <= 128) QIL_TILE_CASE(float, 128);
@@ -499,4 +555,24 @@ extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, c
   if (d <= 128) QIL_TILE_CASE(bf16_t, 128);
   QIL_TILE_CASE(bf16_t, 256);
 #undef QIL_TILE_CASE
+}
+
+extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                             const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
+                             void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
+                             int window, float scale, int dtype, hipStream_t s) {
+  return tile_dispatch(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
+                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, nullptr, 0, 0, 1);
+}
+
+extern "C" int qil_attn_tile_in_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                      const int* block_tables, int table_stride, const int* cu_seqlens,
+                                      const int* seq_starts, void* workspace, int total_rows, int n_seqs, int max_query,
+                                      int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
+                                      int parts, int dtype, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if (parts < 2 || P < 64 || P % 64 || !workspace || total_rows < 1) return -1;
+  return tile_dispatch(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, nullptr, n_seqs,
+                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, (float*)workspace, total_rows,
+                       P, parts);
 }

@@ -546,10 +546,16 @@ TILE_KEY_PARTS = None   # tests: (keys per part, parts) forces the tile kernel's
 
 
 def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context):
-    """(keys per part, parts) for the matrix-core tile kernel; parts == 1: the keys in one piece."""
-    if dtype != torch.bfloat16:
-        return 0, 1
+    """(keys per part, parts) for the matrix-core tile kernels; parts == 1: the keys in one piece."""
     part = ctypes.c_int(0)
+    if dtype != torch.bfloat16 or not (head_dim in (64, 128) and
+                                       lib.qil_attn_tile_bf16_takes(head_dim, page_size, table_stride)):
+        parts = lib.qil_attn_tile_key_parts(n_seqs, max_query, heads, kv_heads, head_dim, max_context, _code(dtype),
+                                            ctypes.byref(part))
+        if TILE_KEY_PARTS is not None:
+            part = ctypes.c_int(TILE_KEY_PARTS[0])
+            parts = max(TILE_KEY_PARTS[1], -(-max_context // part.value))
+        return part.value, parts
     parts = lib.qil_attn_tile_parts(n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context,
                                     ctypes.byref(part))
     if TILE_KEY_PARTS is not None and head_dim in (64, 128) and lib.qil_attn_tile_bf16_takes(head_dim, page_size,
@@ -609,11 +615,19 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             merged = n if tile_seqs is None else n - single_rows.shape[0]
             workspace = torch.empty(lib.qil_attn_rows_workspace(merged, heads, head_dim, parts) // 4, dtype=torch.float32,
                                     device=qkv.device)
-            _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
-                                                _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
-                                                _ptr(seq_starts), _ptr(workspace), merged, n_seqs, max_query, heads,
-                                                kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
-                                                parts, _stream()), 'attn_tile_parts')
+            if qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
+                    lib.qil_attn_tile_bf16_takes(head_dim, page_size, block_tables.shape[1]):
+                _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                                                    _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
+                                                    _ptr(seq_starts), _ptr(workspace), merged, n_seqs, max_query, heads,
+                                                    kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
+                                                    parts, _stream()), 'attn_tile_parts')
+            else:
+                _check(lib.qil_attn_tile_in_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
+                                                  _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
+                                                  _ptr(seq_starts), _ptr(workspace), merged, n_seqs, max_query, heads,
+                                                  kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
+                                                  parts, _code(qkv.dtype), _stream()), 'attn_tile_in_parts')
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), merged, heads, head_dim,
                                       int(window or 0), part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:

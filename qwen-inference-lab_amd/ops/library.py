@@ -180,6 +180,10 @@ def _declare(lib):
     lib.qil_attn_tile_parts.restype = i
     lib.qil_attn_tile_bf16_parts.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, f, i, i, p]
     lib.qil_attn_tile_bf16_parts.restype = i
+    lib.qil_attn_tile_key_parts.argtypes = [i, i, i, i, i, i, i, ctypes.POINTER(ctypes.c_int)]
+    lib.qil_attn_tile_key_parts.restype = i
+    lib.qil_attn_tile_in_parts.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_tile_in_parts.restype = i
     lib.qil_attn_tile_waves.argtypes = [i]
     lib.qil_attn_tile_waves.restype = None
     lib.qil_gemm_bf16_streams.argtypes = [i, i, i, i]

@@ -891,6 +891,39 @@ def test_prompt_portion_with_keys_in_parts(ops, monkeypatch, lengths, chunks, d,
     mixed_attention_case(ops, torch.bfloat16, lengths, chunks, 16, d, heads, kv_heads, window, scale=d ** -0.5)
 
 
+@pytest.mark.parametrize('dtype,lengths,chunks,page_size,d,heads,kv_heads,window,split', [
+    (torch.float32, [700, 90, 33], [100, 1, 33], 16, 128, 16, 4, None, (64, 2)),    # parts of two float32 tiles
+    (torch.float32, [513, 200, 64], [70, 200, 1], 16, 128, 16, 8, None, (128, 2)),  # a part's edge inside a portion's rows
+    (torch.float32, [640], [129], 8, 64, 4, 2, None, (192, 2)),                     # a portion that starts on an edge
+    (torch.float32, [600, 64], [77, 17], 4, 40, 10, 2, 100, (64, 3)),               # d = 40, g = 5, a window
+    (torch.float32, [900], [2], 16, 256, 2, 2, 300, (256, 2)),                      # two rows, g = 1, d = 256
+    (torch.bfloat16, [1030, 300], [130, 2], 16, 96, 6, 2, 64, (64, 4)),             # bfloat16 of a head size without a kernel of its own
+    (torch.bfloat16, [700, 40], [300, 40], 3, 128, 8, 4, None, (128, 2)),           # ... or of pages of 3 keys
+])
+def test_prompt_portion_with_keys_in_parts_on_the_general_kernel(ops, monkeypatch, dtype, lengths, chunks, page_size, d,
+                                                                 heads, kv_heads, window, split):
+    """The float32 path, and bfloat16 sizes without a kernel of their own, cut a portion's keys into parts on the
+    general tile kernel; forced on short contexts here, against float64."""
+    monkeypatch.setattr(ops, 'TILE_KEY_PARTS', split)
+    mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, window, scale=d ** -0.5)
+
+
+@pytest.mark.parametrize('dtype,d,page_size', [(torch.float32, 128, 16), (torch.float32, 64, 16), (torch.bfloat16, 96, 16)])
+@pytest.mark.parametrize('lengths,chunks,heads,kv_heads,window', [
+    ([2048], [128], 16, 8, None),
+    ([3000] + [900] * 6, [128] + [1] * 6, 8, 2, None),          # one portion beside decoded rows
+    ([2500], [130], 8, 2, 1100),
+])
+def test_general_tile_kernel_deep_in_a_long_context(ops, dtype, d, page_size, lengths, chunks, heads, kv_heads, window):
+    """The sizes at which the general kernel's split is chosen by itself."""
+    lib = ops.library.load()
+    table_stride = -(-max(lengths) // page_size)
+    part, parts = ops.tile_key_parts(lib, dtype, sum(c > 1 for c in chunks), max(chunks), heads, kv_heads, d, page_size,
+                                     table_stride, max(lengths))
+    assert parts > 1 and part % 64 == 0 and part * parts >= max(lengths)
+    mixed_attention_case(ops, dtype, lengths, chunks, page_size, d, heads, kv_heads, window, scale=d ** -0.5)
+
+
 @pytest.mark.parametrize('lengths,chunks,heads,kv_heads,window', [
     ([2048], [128], 32, 8, None),
     ([4000, 3000, 1500], [64, 1, 2], 16, 8, None),
