@@ -1057,6 +1057,38 @@ def test_prompt_kernels_find_one_key_at_the_edges_of_tiles_and_parts(ops, monkey
     torch.testing.assert_close(got.float().cpu(), values_of(histories, row_seq, targets, heads, kv_heads), atol=1e-6, rtol=0)
 
 
+@pytest.mark.parametrize('dtype,d,page_size', [(torch.float32, 128, 16), (torch.float32, 40, 4), (torch.bfloat16, 96, 16)])
+@pytest.mark.parametrize('length,chunk,split', [(700, 100, (64, 2)), (300, 300, None), (2048, 128, None)])
+def test_general_tile_kernel_finds_one_key_at_the_edges_of_tiles_and_parts(ops, monkeypatch, dtype, d, page_size, length,
+                                                                         chunk, split):
+    """The general tile kernel (float32; bfloat16 sizes without a kernel of their own), keys in one piece or in
+    parts that are merged: every row aims at one key, in turn the first, the ends of 32- and 64-key tiles and of
+    the parts, its own key and the one before it."""
+    heads, kv_heads = 4, 2
+    if split is not None:
+        monkeypatch.setattr(ops, 'TILE_KEY_PARTS', split)
+    k_cache, v_cache, table, histories = build_cache([length], page_size, kv_heads, d, dtype)
+    start = length - chunk
+    fixed = [0, 31, 32, 63, 64, 127, 128, 191, 192, 255, 256]
+    targets = []
+    for i in range(chunk):
+        position = start + i
+        choices = [t for t in fixed + [start - 1, start] if 0 <= t <= position] + [position, max(position - 1, 0)]
+        targets.append(choices[i % len(choices)])
+    row_seq = [0] * chunk
+    q = pointed_queries(histories, row_seq, targets, heads, kv_heads, d, dtype)
+    dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
+    if split is None and length > 1000:
+        part, parts = ops.tile_key_parts(ops.library.load(), dtype, 1, chunk, heads, kv_heads, d, page_size,
+                                         table.shape[1], length)
+        assert parts > 1 and part in (128, 192, 256), 'a portion deep in a context: the split is chosen by itself'
+    got = ops.paged_attention(q, heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache,
+                              page_size=page_size, block_tables=table, row_seq=dev(row_seq),
+                              positions=dev(list(range(start, length))), cu_seqlens=dev([0, chunk]), seq_starts=dev([start]),
+                              single_rows=dev([]), n_seqs=1, max_query=chunk, max_context=length, scale=1.0, window=None)
+    torch.testing.assert_close(got.float().cpu(), values_of(histories, row_seq, targets, heads, kv_heads), atol=1e-6, rtol=0)
+
+
 def test_sampling(ops):
     vocab = 151936
     logits = rand(5, vocab, scale=2.0)
