@@ -35,6 +35,17 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// The sum of every aligned group of 2^log2 consecutive lanes (up to 32), in all of its lanes: the same moves, as
+// many as the group needs, and one exchange between the two rows of 16 for groups of 32.
+__device__ __forceinline__ float group_sum(float v, int log2) {
+  if (log2 >= 1) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  if (log2 >= 2) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+  if (log2 >= 3) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+  if (log2 >= 4) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+  if (log2 >= 5) v += __shfl_xor(v, 16, QIL_WAVE);
+  return v;
+}
+
 template <typename T, int GT>
 __global__ void __launch_bounds__(ATT_THREADS)
 attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
@@ -62,8 +73,8 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
   const int* table = block_tables + (size_t)row_seq[row] * table_stride;
 
   float* scores = lds;                            // [GT][P]
-  float* reduce = lds + GT * P;                   // [16] block reductions
-  float* wave_acc = reduce + 16;                  // [ATT_WAVES][GT][d]
+  float* reduce = lds + GT * P;                   // [2][ATT_WAVES][GT] the waves' maxima and sums
+  float* wave_acc = reduce + 64;                  // [ATT_WAVES][GT][d]
 
   for (int h0 = 0; h0 < g; h0 += GT) {
     // ---- scores of this head tile against the block's keys
@@ -99,31 +110,47 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
           float dot = 0.f;
 #pragma unroll
           for (int e = 0; e < 8; ++e) dot += qv[h][e] * kv[u][e];
-          for (int o = TG >> 1; o > 0; o >>= 1) dot += __shfl_xor(dot, o, QIL_WAVE);
+          dot = group_sum(dot, tg_log2);
           if (sub == 0 && t < count) scores[h * P + t] = dot * scale;
         }
       }
     }
     __syncthreads();
 
-    // ---- softmax statistics per head (block wide), probabilities back into LDS
+    // ---- softmax statistics per head (block wide), probabilities back into LDS: the tile's heads together, the
+    // waves' maxima and sums meeting in LDS in wave order (three barriers a tile of heads, not four a head)
     float m_h[GT], l_h[GT];
 #pragma unroll
     for (int h = 0; h < GT; ++h) {
       float m = -INFINITY;
       for (int t = threadIdx.x; t < count; t += ATT_THREADS) m = fmaxf(m, scores[h * P + t]);
-      m = block_max(m, reduce);
+      m = wave_max(m);
+      if (lane == 0) reduce[wave * GT + h] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      float m = reduce[h];
+#pragma unroll
+      for (int w = 1; w < ATT_WAVES; ++w) m = fmaxf(m, reduce[w * GT + h]);
       float l = 0.f;
       for (int t = threadIdx.x; t < count; t += ATT_THREADS) {
         const float p = expf(scores[h * P + t] - m);
         scores[h * P + t] = p;
         l += p;
       }
-      l = block_sum(l, reduce);
+      l = wave_sum(l);
+      if (lane == 0) reduce[(ATT_WAVES + wave) * GT + h] = l;
       m_h[h] = m;
-      l_h[h] = l;
     }
     __syncthreads();
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      float l = 0.f;
+#pragma unroll
+      for (int w = 0; w < ATT_WAVES; ++w) l += reduce[(ATT_WAVES + w) * GT + h];      // fixed order
+      l_h[h] = l;
+    }
 
     // ---- weighted values.  V is [pages, kv_heads, d, page_size]: a key's elements lie page_size apart and the keys
     // of a page side by side, so here a wave's lanes are 16 consecutive keys x 4 chunks of 8 elements (a load
@@ -266,7 +293,7 @@ static int next_pow2_log2(int v) {
 }
 
 // LDS floats the partial kernel needs.
-static size_t rows_lds_floats(int gt, int P, int d) { return (size_t)gt * P + 16 + (size_t)ATT_WAVES * gt * d; }
+static size_t rows_lds_floats(int gt, int P, int d) { return (size_t)gt * P + 64 + (size_t)ATT_WAVES * gt * d; }
 
 template <typename T>
 static int launch_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
