@@ -202,7 +202,10 @@ def main():
     step_s, contexts = decode_run(args.batch)
     note(f'decode batch {args.batch}: {step_s * 1e3:.3f} ms/step')
     if args.phase == 'decode':
-        print(json.dumps({'decode_ms_per_step': round(step_s * 1e3, 4), 'batch': args.batch, 'layers': args.layers}))
+        achieved = decode_bytes(config, element, contexts) / step_s / 1e9
+        print(json.dumps({'decode_ms_per_step': round(step_s * 1e3, 4), 'batch': args.batch, 'layers': args.layers,
+                          'tokens_per_s': round(args.batch / step_s, 1), 'hbm_gb_per_s': round(achieved, 1),
+                          'hbm_frac': round(achieved / HBM_GBPS, 4)}))
         return 0
     points = {}
     for batch in [int(b) for b in args.points.split(',') if b]:
