@@ -7,6 +7,7 @@
 // have K contiguous (nn.Linear layout, qil/model.py:32-40).  The tiled kernel: 64 x 64 x 16 tiles in
 // LDS, 256 threads, 4 x 4 outputs a thread.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 #include "merge_parts.h"
@@ -321,6 +322,160 @@ gemm_f32_lines_kernel(const float* __restrict__ A, UnmergedA unmerged, GatedA ga
   }
 }
 
+// 17 to 64 rows, K split into ranges of whole stages: the whole-line kernel with A passing through LDS a stage (64
+// columns) at a time, in two slots that the block's threads fill in turn from registers loaded three stages ahead,
+// as W's are (the scheme of gemm_bf16_chunks_kernel in gemm_bf16.hip).  One barrier a stage.  MT: 16-row tiles of A;
+// every W fragment read from the wave's buffer serves MT products.  With 64 rows the matrix cores allow 4.9 TB/s of
+// weights (32 products of 16 x 16 x 4 a stage and row tile), about what memory gives.
+#define FC_ROW (FL_STAGE + FL_PAD)
+#define FC_MOST_ROWS 64
+
+template <int MT>
+__global__ void __launch_bounds__(FL_WAVES * QIL_WAVE)
+gemm_f32_chunks_kernel(const float* __restrict__ A, const float* __restrict__ W, float* __restrict__ C, int M, int N,
+                       int K, int cols_per_split) {
+  extern __shared__ __align__(16) float fc_lds[];           // two stages of A [16 MT][64 + pad], then the waves' buffers
+  constexpr int A_ROWS = 16 * MT, SLOT = A_ROWS * FC_ROW;
+  constexpr int PIECES = A_ROWS * 16 / (FL_WAVES * QIL_WAVE);     // 16-byte pieces of a stage of A per thread
+  static_assert(PIECES >= 1, "a stage of A has fewer pieces than the block has threads");
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int r = lane & 15, kb = lane >> 4;
+  const int split = blockIdx.z;
+  const int n0 = (blockIdx.x * FL_WAVES + wave) * 16;
+  const int k_begin = split * cols_per_split, stages = cols_per_split / FL_STAGE;
+  float* buffer = fc_lds + 2 * SLOT + wave * (16 * FL_STAGE);
+
+  const int load_row = lane >> 4, piece = lane & 15;
+  const float* source[4];                                  // rows past N read a valid row and are never stored
+  int place[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int row = 4 * u + load_row;
+    source[u] = W + (size_t)min(n0 + row, N - 1) * K + k_begin + piece * 4;
+    place[u] = row * FL_STAGE + ((piece ^ row) & 15) * 4;
+  }
+  // This thread's pieces of a stage of A.  Rows past M read row M - 1: their products land in rows of the result
+  // that are never stored (a load under a condition would make the compiler wait for every load in flight).
+  const float* a_source[PIECES];
+  int a_place[PIECES];
+#pragma unroll
+  for (int u = 0; u < PIECES; ++u) {
+    const int p = threadIdx.x + u * (FL_WAVES * QIL_WAVE), row = p >> 4, pc = p & 15;
+    a_source[u] = A + (size_t)min(row, M - 1) * K + k_begin + pc * 4;
+    a_place[u] = row * FC_ROW + pc * 4;
+  }
+  const int turn = blockIdx.x % stages;
+  auto column = [&](int stage) { const int st = stage + turn; return (st >= stages ? st - stages : st) * FL_STAGE; };
+  f32x4v w0[4], w1[4], w2[4], a0[PIECES], a1[PIECES], a2[PIECES];
+  auto request = [&](f32x4v (&stage_w)[4], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) stage_w[u] = *reinterpret_cast<const f32x4v*>(source[u] + at);
+  };
+  auto request_a = [&](f32x4v (&stage_a)[PIECES], int stage) {
+    const int at = column(stage);
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) stage_a[u] = *reinterpret_cast<const f32x4v*>(a_source[u] + at);
+  };
+  auto store_a = [&](const f32x4v (&stage_a)[PIECES], int stage) {
+    float* slot = fc_lds + (stage & 1) * SLOT;
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) *reinterpret_cast<f32x4v*>(slot + a_place[u]) = stage_a[u];
+  };
+  request_a(a0, 0); request_a(a1, 1); request_a(a2, 2);     // the host sees to stages >= 3
+  request(w0, 0); request(w1, 1); request(w2, 2);
+  store_a(a0, 0);
+  if (3 < stages) request_a(a0, 3);
+  __syncthreads();
+
+  f32x4v acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+  auto pass = [&](const f32x4v (&stage_w)[4]) {            // registers -> buffer
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<f32x4v*>(buffer + place[u]) = stage_w[u];
+  };
+  auto multiply = [&](int stage) {
+    const float* a_row = fc_lds + (stage & 1) * SLOT + r * FC_ROW + kb * 4;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {                        // columns 16 s4 + 4 kb .. + 3 of the stage: four products a tile
+      const f32x4v b = *reinterpret_cast<const f32x4v*>(buffer + r * FL_STAGE + (((4 * s4 + kb) ^ r) & 15) * 4);
+      f32x4v a[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) a[t] = *reinterpret_cast<const f32x4v*>(a_row + t * 16 * FC_ROW + s4 * 16);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)                           // the tiles in turn: a product never waits for the one before it
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][c], b[c], acc[t], 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  // Stage s: its W goes from registers w to the buffer; registers a hold stage s + 1 of A.  `inner`: every request
+  // of the stage has a target (a request under a condition, even a uniform one, makes the compiler wait for all
+  // loads in flight at the next use of any of them, so the stages that need conditions are apart).
+  auto step = [&](int s, f32x4v (&w)[4], f32x4v (&a)[PIECES], auto inner) {
+    pass(w);
+    if (decltype(inner)::value || s + 3 < stages) request(w, s + 3);
+    if (decltype(inner)::value || s + 1 < stages) store_a(a, s + 1);
+    if (decltype(inner)::value || s + 4 < stages) request_a(a, s + 4);
+    multiply(s);
+    __syncthreads();
+  };
+  int s = 0;
+  for (; s + 7 <= stages; s += 3) {
+    step(s, w0, a1, std::true_type());
+    step(s + 1, w1, a2, std::true_type());
+    step(s + 2, w2, a0, std::true_type());
+  }
+  for (; s + 3 <= stages; s += 3) {
+    step(s, w0, a1, std::false_type());
+    step(s + 1, w1, a2, std::false_type());
+    step(s + 2, w2, a0, std::false_type());
+  }
+  if (s < stages) step(s, w0, a1, std::false_type());
+  if (s + 1 < stages) step(s + 1, w1, a2, std::false_type());
+  float* out = C + (size_t)split * M * N;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = t * 16 + 4 * kb + i, n = n0 + r;
+      if (m < M && n < N) out[(size_t)m * N + n] = acc[t][i];
+    }
+}
+
+static bool fc_takes(int M, int N, int K, int splits) {
+  return M > 16 && M <= FC_MOST_ROWS && N >= 1 && splits >= 1 && K % (FL_STAGE * splits) == 0 &&
+         K / (FL_STAGE * splits) >= FL_DEPTH;
+}
+
+// K splits of that kernel: the most (a power of two up to 8, with at least three stages each) that keep the blocks
+// within the 256 CUs (the rule of the bfloat16 kernel of the same shape).
+static int fc_splits(int M, int N, int K) {
+  if (!fc_takes(M, N, K, 1)) return 0;
+  const long tiles = (N + 16 * FL_WAVES - 1) / (16 * FL_WAVES);
+  int splits = 1;
+  for (int c = 2; c <= 8; c *= 2)
+    if (tiles * c <= 256 && fc_takes(M, N, K, c)) splits = c;
+  return splits;
+}
+
+template <int MT>
+static int launch_f32_chunks(const float* A, const float* W, float* C, int M, int N, int K, int splits, hipStream_t s) {
+  const size_t lds = ((size_t)2 * 16 * MT * FC_ROW + (size_t)FL_WAVES * 16 * FL_STAGE) * sizeof(float);
+  auto kernel = gemm_f32_chunks_kernel<MT>;
+  static size_t granted = 0;                              // per instantiation
+  if (lds > 64 * 1024 && lds > granted) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    granted = lds;
+  }
+  dim3 grid((N + 16 * FL_WAVES - 1) / (16 * FL_WAVES), 1, splits);
+  hipLaunchKernelGGL(kernel, grid, dim3(FL_WAVES * QIL_WAVE), lds, s, A, W, C, M, N, K, K / splits);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
 static size_t fl_lds_bytes(int M, int K, int splits) {
   return ((size_t)(M <= 8 ? 8 : 16) * (K / splits + FL_PAD) + (size_t)FL_WAVES * 16 * FL_STAGE) * sizeof(float);
 }
@@ -428,6 +583,7 @@ extern "C" int qil_gemm_f32_splits(int M, int N, int K) {
   }
   if (K % 4) return 1;
   if (const int lines = fl_splits(M, N, K)) return lines;
+  if (const int chunks = fc_splits(M, N, K)) return chunks;
   const int column_blocks = (N + 127) / 128, steps = (K + 15) / 16;
   int sp = (768 + column_blocks - 1) / column_blocks;
   if (sp > 8) sp = 8;
@@ -448,6 +604,8 @@ extern "C" int qil_gemm_f32(const float* A, const float* W, const float* bias, f
   if (splits > 1 && (!stream_ok || bias)) return -1;
   if (stream_ok && !bias && (splits == 1 || splits == fl_splits(M, N, K)) && fl_takes(M, N, K, splits))
     return launch_f32_lines<0>(A, UnmergedA(), GatedA(), W, C, M, N, K, splits, s);
+  if (stream_ok && !bias && fc_takes(M, N, K, splits) && (splits == 1 || splits == fc_splits(M, N, K)))
+    return M <= 32 ? launch_f32_chunks<2>(A, W, C, M, N, K, splits, s) : launch_f32_chunks<4>(A, W, C, M, N, K, splits, s);
   if (stream_ok) {
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;           // 16-row tiles of A a block keeps
     const int steps = (K + 15) / 16, steps_per_split = (steps + splits - 1) / splits;
