@@ -220,8 +220,6 @@ def test_first_tokens_of_a_sequence(case):
 def test_long_decoding_crosses_attention_splits(case):
     """Single tokens up to a context longer than one attention split (256 keys)."""
     config, weights, model, page_size = case
-    if config is not plain.TINY_A:
-        pytest.skip('one configuration is enough for the long run')
     tokens = tokens_for(config, 300, 44)
     runner = ModelRunner(model, num_pages=-(-300 // page_size), page_size=page_size)
     poison(runner)
