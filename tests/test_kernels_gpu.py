@@ -125,6 +125,25 @@ def test_linear_float32_whole_lines(ops, m, k):
         torch.testing.assert_close(alone.tensor[:, 0], got.tensor[:, m - 1], atol=0, rtol=0)
 
 
+@pytest.mark.parametrize('k', [192, 256, 320, 384, 448, 512, 576, 640, 704, 1024, 4096])
+@pytest.mark.parametrize('m', [17, 32, 33, 48, 64])
+def test_linear_float32_whole_lines_of_17_to_64_rows(ops, m, k):
+    """The float32 product of 17 to 64 rows with A passing through LDS a stage at a time: every number of stages from
+    3 on (the first stages in an unrolled loop of three, the last ones apart), two or four row tiles, rows of W past the
+    end of a wave's sixteen and of a block's 128, whole and split over K; a row's result does not depend on how many
+    rows come after it."""
+    n = 130 if k != 1024 else 2100
+    x, w = rand(m, k), rand(n, k, seed=1, scale=k ** -0.5)
+    want = x.double() @ w.double().t()
+    check(ops.linear(x, w, None), want, torch.float32, scale=4)
+    got = ops.linear(x, w, None, partials=True)
+    check(got.sum() if isinstance(got, ops.Partials) else got, want, torch.float32, scale=4)
+    fewer = ops.linear(x[:17].contiguous(), w, None, partials=True)
+    tensor = lambda r: r.tensor if isinstance(r, ops.Partials) else r[None]
+    assert tensor(fewer).shape[0] == tensor(got).shape[0]
+    torch.testing.assert_close(tensor(fewer), tensor(got)[:, :17], atol=0, rtol=0)
+
+
 @pytest.mark.parametrize('m,n,k', [(3, 1024, 4096), (16, 300, 2048), (20, 4096, 4096), (64, 1024, 3072), (33, 130, 516),
                                    (48, 2000, 100), (65, 512, 1024), (128, 4096, 1024), (160, 6144, 4096)])
 def test_linear_float32_partial_sums(ops, m, n, k):
