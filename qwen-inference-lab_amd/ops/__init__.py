@@ -483,8 +483,27 @@ def _rows_part(rows, kv_heads, max_context):
 
 
 def _decode_parts(rows, kv_heads, max_context):
-    """(keys a part, parts) of the matrix-core decode kernel: the context is split until the chip has enough blocks."""
-    wanted = max(1, DECODE_BLOCKS // (rows * kv_heads))
+    """(keys a part, parts) of the matrix-core decode kernel: the context is split until the chip has enough blocks.
+
+    With more blocks than CUs the blocks run in rounds, and a last round that is mostly empty costs a whole one (33
+    rows of 8 kv heads are 264 blocks: 75 us against 52 for 32 rows of 2,048 keys).  Then the context is cut so that
+    the rounds fill: the fewest parts of 1,024 keys or more that fill their rounds to 90 %, else of 512 or more to
+    80 % (33 rows: 4 parts, 69 us; at 8,192 keys 7 parts, about 197 against 276; 65 rows 2 parts, 112 against 116)."""
+    blocks = rows * kv_heads
+    if blocks > DECODE_BLOCKS:
+        fill = lambda count: count / (-(-count // DECODE_BLOCKS) * DECODE_BLOCKS)
+        if fill(blocks) < 0.72:
+            for fewest_keys, enough in ((1024, 0.9), (512, 0.8)):
+                for parts in range(2, 33):
+                    part = -(-(-(-max_context // parts)) // 64) * 64
+                    if part < fewest_keys:
+                        break
+                    if part > DECODE_MAX_PART:
+                        continue
+                    actual = -(-max_context // part)
+                    if fill(blocks * actual) >= enough:
+                        return part, actual
+    wanted = max(1, DECODE_BLOCKS // blocks)
     part = min(DECODE_MAX_PART, max(DECODE_MIN_PART, -(-(-(-max_context // wanted)) // 64) * 64))
     return part, max(1, -(-max_context // part))
 

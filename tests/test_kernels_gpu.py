@@ -635,6 +635,31 @@ def test_decode_rows_against_float64(ops, dtype, lengths, page_size, d, heads, k
         torch.testing.assert_close(ops.paged_attention(qkv, **args)[0], got[0], atol=0, rtol=0)
 
 
+def test_decode_rows_with_parts_that_fill_the_rounds(ops):
+    """33 rows of 8 kv heads are more blocks than CUs: the matrix-core decode kernel then cuts the contexts into four
+    parts; against float64, with contexts that end in every part."""
+    dtype, page_size, d, heads, kv_heads = torch.bfloat16, 16, 128, 16, 8
+    lengths = [2048 - 61 * i for i in range(33)]
+    assert ops._decode_parts(len(lengths), kv_heads, max(lengths)) == (512, 4)
+    k_cache, v_cache, table, histories = build_cache(lengths, page_size, kv_heads, d, dtype)
+    rows = len(lengths)
+    qkv = rand(rows, heads * d, dtype=dtype)
+    args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, k_cache=k_cache, v_cache=v_cache, page_size=page_size,
+                block_tables=table, row_seq=torch.arange(rows, dtype=torch.int32).cuda(),
+                positions=torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda(), cu_seqlens=None,
+                seq_starts=None, single_rows=None, n_seqs=rows, max_query=1, max_context=max(lengths), scale=d ** -0.5,
+                window=None)
+    got = ops.paged_attention(qkv, **args)
+    expected = []
+    for row, (k, v) in enumerate(histories):
+        q = qkv[row].reshape(heads, d).double().cpu()
+        kh = k.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
+        vh = v.double().repeat_interleave(heads // kv_heads, dim=1).transpose(0, 1)
+        score = (q[:, None, :] * kh).sum(-1) * d ** -0.5
+        expected.append((score.softmax(-1)[..., None] * vh).sum(1).reshape(-1))
+    torch.testing.assert_close(got.double().cpu(), torch.stack(expected), **ATT_TOL[dtype])
+
+
 @pytest.mark.parametrize('lengths,window,d,heads,kv_heads,out_features', [
     ([2100, 1, 700, 1290, 64, 2047, 300, 1500], None, 128, 32, 8, 4096),
     ([900, 2100, 33], 500, 128, 32, 4, 300),

@@ -25,3 +25,22 @@ def test_decode_parts_cover_the_context():
         part, parts = ops._decode_parts(rows, kv_heads, context)
         assert part % 64 == 0 and ops.DECODE_MIN_PART <= part <= ops.DECODE_MAX_PART
         assert parts >= 1 and part * parts >= context and part * (parts - 1) < context
+
+
+def test_decode_parts_fill_their_rounds_of_blocks():
+    """More blocks than CUs run in rounds: where one part a row would leave the last round mostly empty the context
+    is cut so that the rounds fill; where the rounds are full anyway, or the context is short, it stays whole."""
+    kv_heads = 8
+    assert ops._decode_parts(32, kv_heads, 2048) == (2048, 1)         # 256 blocks: one round
+    assert ops._decode_parts(33, kv_heads, 2048) == (512, 4)          # 264 blocks -> 1,056: 5 rounds, 82 % full
+    assert ops._decode_parts(40, kv_heads, 2048) == (1024, 2)
+    assert ops._decode_parts(48, kv_heads, 2048) == (2048, 1)         # 384 blocks: the second round is half full
+    assert ops._decode_parts(64, kv_heads, 2048) == (2048, 1)
+    assert ops._decode_parts(65, kv_heads, 2048) == (1024, 2)
+    assert ops._decode_parts(33, kv_heads, 8192) == (1216, 7)         # long parts: filled to 90 %
+    assert ops._decode_parts(33, kv_heads, 700) == (704, 1)           # too short to cut
+    for rows in range(1, 300, 7):
+        for context in (1, 300, 2048, 5000, 40000, 131072):
+            part, parts = ops._decode_parts(rows, kv_heads, context)
+            assert part % 64 == 0 and ops.DECODE_MIN_PART <= part <= ops.DECODE_MAX_PART
+            assert parts >= 1 and part * parts >= context and part * (parts - 1) < context
