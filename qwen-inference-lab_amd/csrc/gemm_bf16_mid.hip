@@ -30,7 +30,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define MID_STAGE 64                                       // columns of K a stage: rows of 128 bytes
 #define MID_WAVES 4
 #define MID_COLS (32 * MID_WAVES)                          // columns of C a block
-#define MID_MOST_ROWS 256
+#define MID_MOST_ROWS 256                                 // rows of a block
+#define MID_MOST_ROWS_IN_BLOCKS 1024                      // rows of a product: up to four blocks of rows
 #define MID_LDS_LIMIT (156 * 1024)
 // Starting stages of the blocks of a product whose K is not split (split parts read different bands already).
 // Measured at Qwen3-8B's gate/up sizes, 40 / 96 / 160 rows: 44 / 46 / 54 us with 1, 38 / 41 / 51 with 4 and with 16;
@@ -55,9 +56,12 @@ __host__ __device__ constexpr int mid_a_ring(int mt) {
 // in LDS) and loads that are sent far ahead (W, from memory) belong to different waves.
 template <int MT, typename OUT, bool GATED>
 __global__ void __launch_bounds__((MID_WAVES + 1) * QIL_WAVE, 1)
-gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M, int N, int K,
+gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, OUT* __restrict__ C, int M_all, int N, int K,
                      int stages, int waves, int turns) {
   constexpr int RW = mid_w_ring(MT), RA = mid_a_ring(MT);
+  // more than 32 MT rows: grid.z counts blocks of 32 MT rows, each a product of its own over the same W
+  const int row0 = blockIdx.z * (32 * MT), M = min(M_all - row0, 32 * MT);
+  A += (size_t)row0 * K;
   constexpr int W_SLOT = MID_WAVES * 4096, A_SLOT = MT * 4096;   // bytes of a stage: 32 rows x 128 bytes a wave; 32 MT rows
   extern __shared__ __align__(1024) unsigned char lds[];   // W ring, then A ring
   unsigned char* a_ring = lds + RW * W_SLOT;
@@ -168,7 +172,7 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
     for (int t = 0; t < MT; ++t) {
       const int m = 32 * t + l32;
       if (m >= M) continue;
-      OUT* row = C + (size_t)m * inner + n0 / 2 + 4 * half;
+      OUT* row = C + (size_t)(row0 + m) * inner + n0 / 2 + 4 * half;
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
         float v[4];
@@ -183,7 +187,7 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
     }
     return;
   }
-  OUT* out = C + (size_t)blockIdx.y * M * N;
+  OUT* out = C + ((size_t)blockIdx.y * M_all + row0) * N;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 32 * t + l32;
@@ -205,14 +209,15 @@ gemm_bf16_mid_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
 // whole stages, 4 stages or more a split and at most 16 splits, the one with the least time by this count (rounds
 // times a block's stages, a little for every split's partial sums) is taken; splits: 0 = free, else given.
 static bool mid_plan(int M, int N, int K, int* waves, int* splits) {
-  if (M < 1 || M > MID_MOST_ROWS || N < 32 || N % 32 || K < 4 * MID_STAGE || K % MID_STAGE) return false;
+  if (M < 1 || M > MID_MOST_ROWS_IN_BLOCKS || N < 32 || N % 32 || K < 4 * MID_STAGE || K % MID_STAGE) return false;
   const int stages = K / MID_STAGE, given = *splits;
+  const int row_blocks = (M + MID_MOST_ROWS - 1) / MID_MOST_ROWS;
   double best = 0;
   bool found = false;
   for (int w = MID_WAVES; w >= 2; --w)
     for (int sp = 1; sp <= 16; ++sp) {
       if ((given && sp != given) || stages % sp || stages / sp < 4) continue;
-      const long blocks = (long)((N / 32 + w - 1) / w) * sp;
+      const long blocks = (long)((N / 32 + w - 1) / w) * sp * row_blocks;
       const long rounds = (blocks + 255) / 256;
       // a block's time: its stages, each as long as its W takes at the CU's share of the memory's rate, but not
       // shorter than what a stage costs anyway (barrier, sending the loads, the first fragments); CUs without a block
@@ -234,7 +239,7 @@ static int mid_launch(const void* A, const void* W, void* C, int M, int N, int K
     if (e != hipSuccess) return (int)e;
     granted = true;
   }
-  dim3 grid((N / 32 + waves - 1) / waves, splits);
+  dim3 grid((N / 32 + waves - 1) / waves, splits, (M + 32 * MT - 1) / (32 * MT));
   hipLaunchKernelGGL(kernel, grid, dim3((waves + 1) * QIL_WAVE), lds, s, (const bf16_t*)A, (const bf16_t*)W, (OUT*)C, M, N, K,
                      K / MID_STAGE / splits, waves, splits == 1 ? MID_TURNS : 1);
   QIL_RETURN_LAUNCH_STATUS();
@@ -247,7 +252,9 @@ static int mid_dispatch(const void* A, const void* W, void* C, int M, int N, int
   case MT:                                                                                                    \
     return out_dtype == QIL_F32 ? mid_launch<MT, float, GATED>(A, W, C, M, N, K, waves, splits, s)            \
                                 : mid_launch<MT, bf16_t, GATED>(A, W, C, M, N, K, waves, splits, s)
-  switch ((M + 31) / 32) {
+  // more than 256 rows: blocks of rows of equal size (300 rows: two of 160)
+  const int row_blocks = (M + MID_MOST_ROWS - 1) / MID_MOST_ROWS;
+  switch (((M + 31) / 32 + row_blocks - 1) / row_blocks) {
     QIL_MID_CASE(1);
     QIL_MID_CASE(2);
     QIL_MID_CASE(3);
@@ -269,7 +276,25 @@ int qil_gemm_bf16_mid_splits(int M, int N, int K) {
   return mid_plan(M, N, K, &waves, &splits) ? splits : 0;
 }
 
-// C = A[M, K] W[N, K]^T for 1 <= M <= 256.  splits > 1: C float32 [splits][M][N] partial sums (out_dtype QIL_F32);
+// 1 if a product of 257 to 1,024 rows should run here, in blocks of rows that each stream W again, rather than in the
+// GPU BLAS.  Measured on the GPU alone (replayed graphs), us here against the library, for q/k/v, attention output,
+// gate/up and down: 0.6B sizes 300 rows 10.8 / 7.7 / 11.7 / 8.7 against 10.4 / 9.7 / 10.7 / 12.2, 512 rows 13.9 / 10.4 /
+// 15.4 / 12.3 against 11.0 / 9.8 / 13.4 / 12.6; 8B sizes 300 rows 27.9 / 20.0 / 111 / 48.5 against 29.9 / 26.2 / 76 /
+// 69.7, 512 rows 40.0 / 28.5 / 143 / 69.2 against 39.3 / 30.0 / 91 / 82.3, 768 rows 68 / 41 / 204 / 116 against 51 / 35 /
+// 151 / 96.  What the library is slow at is the long K of few columns (down) up to 512 rows, and everything but the
+// widest products up to some 300 rows.  (A step launched kernel by kernel gains more, the host spending 18 us on a
+// library product against 6 here: 0.6B sizes, 512 rows, 13.6 / 10.0 / 15.1 / 11.9 against 19.5 / 19.2 / 19.5 / 19.9.  The
+// choice does not look at how the step is launched: a step and its replayed graph then run the same kernels and
+// give the same bits.)
+int qil_gemm_bf16_mid_rows_takes(int M, int N, int K) {
+  if (M <= MID_MOST_ROWS || M > 512) return 0;
+  if (!((M <= 320 && N <= 6144) || K >= 2 * N)) return 0;
+  int waves = 0, splits = 0;
+  return mid_plan(M, N, K, &waves, &splits);
+}
+
+// C = A[M, K] W[N, K]^T for 1 <= M <= 1,024 (more than 256 rows: in equal blocks of rows, each a block of the grid
+// over the same W).  splits > 1: C float32 [splits][M][N] partial sums (out_dtype QIL_F32);
 // splits == 1: C [M][N] of out_dtype.  splits: 0 = chosen here (qil_gemm_bf16_mid_splits), else a divisor of K / 64
 // that leaves 4 stages or more.
 int qil_gemm_bf16_mid(const void* A, const void* W, void* C, int M, int N, int K, int out_dtype, int splits, hipStream_t s) {
@@ -285,7 +310,7 @@ int qil_gemm_bf16_mid(const void* A, const void* W, void* C, int M, int N, int K
 // give every CU work.
 int qil_gemm_bf16_mid_gated_takes(int M, int inner, int K) {
   int waves = 0, splits = 1;
-  return inner >= 16 && inner % 16 == 0 && mid_plan(M, 2 * inner, K, &waves, &splits) &&
+  return M <= MID_MOST_ROWS && inner >= 16 && inner % 16 == 0 && mid_plan(M, 2 * inner, K, &waves, &splits) &&
          (2 * inner / 32 + waves - 1) / waves >= 192;
 }
 

@@ -347,7 +347,9 @@ def linear(x, weight, bias=None, out_dtype=None, partials=False, add_to=None):
         _check(lib.qil_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), n, o, k, splits, _stream()), 'gemm_f32')
         return Partials(out) if splits > 1 else out[0]
     _code(x.dtype)
-    if MID_GEMM_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS and bias is None and out_dtype == x.dtype:
+    # (beyond 256 rows: in blocks of rows, for the products that the library is slow at; the kernel's file says which)
+    if bias is None and out_dtype == x.dtype and (MID_GEMM_FEWEST_ROWS <= n <= MID_GEMM_MOST_ROWS or
+                                                   (n > MID_GEMM_MOST_ROWS and lib.qil_gemm_bf16_mid_rows_takes(n, o, k))):
         splits = lib.qil_gemm_bf16_mid_splits(n, o, k)
         if splits == 1 or (splits > 1 and partials):
             out = torch.empty((splits, n, o), dtype=torch.float32 if splits > 1 else x.dtype, device=x.device)

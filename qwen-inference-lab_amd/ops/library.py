@@ -203,6 +203,8 @@ def _declare(lib):
     lib.qil_gemm_bf16_mid_splits.argtypes = [i, i, i]
     lib.qil_gemm_bf16_mid_splits.restype = i
     lib.qil_gemm_bf16_mid.argtypes = [p, p, p, i, i, i, i, i, p]
+    lib.qil_gemm_bf16_mid_rows_takes.argtypes = [i, i, i]
+    lib.qil_gemm_bf16_mid_rows_takes.restype = i
     lib.qil_gemm_bf16_mid_gated_takes.argtypes = [i, i, i]
     lib.qil_gemm_bf16_mid_gated_takes.restype = i
     lib.qil_gemm_bf16_mid_gated.argtypes = [p, p, p, i, i, i, i, p]

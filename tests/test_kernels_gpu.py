@@ -371,12 +371,13 @@ def test_gated_linear(ops, m, inner, k, dtype):
         check(ops.silu_mul(y_turns, interleaved=True), ops.silu_mul((x.double() @ w.double().t()).to(dtype)), dtype, scale=0)
 
 
-@pytest.mark.parametrize('m', [1, 31, 33, 65, 96, 128, 129, 160, 161, 200, 256])
+@pytest.mark.parametrize('m', [1, 31, 33, 65, 96, 128, 129, 160, 161, 200, 256, 257, 300, 512, 513, 777, 1024])
 @pytest.mark.parametrize('n,k', [(4096, 4096), (6144, 1024), (96, 256), (160, 4160), (24576, 512), (32, 320)])
 def test_products_of_up_to_256_rows_loaded_straight_into_lds(ops, m, n, k):
-    """The kernel for 65 to 256 rows (it takes fewer too): 32 x 32 x 16 products, W and A loaded straight into LDS, a
-    wave of its own for A, K split over blocks.  Every plan it makes (2 to 4 multiplying waves, 1 to 16 splits)
-    and forced splits, partial sums and direct results in both types, against float64; and through the op."""
+    """The kernel for 65 to 256 rows (it takes fewer too, and up to 1,024 in equal blocks of rows): 32 x 32 x 16
+    products, W and A loaded straight into LDS, a wave of its own for A, K split over blocks.  Every plan it makes (2
+    to 4 multiplying waves, 1 to 16 splits) and forced splits, partial sums and direct results in both types, against
+    float64; and through the op."""
     lib = ops.library.load()
     x = rand(m, k, dtype=torch.bfloat16)
     w = rand(n, k, dtype=torch.bfloat16, seed=1, scale=2.0 * k ** -0.5)
@@ -407,7 +408,12 @@ def test_products_of_up_to_256_rows_loaded_straight_into_lds(ops, m, n, k):
 
 def test_products_of_up_to_256_rows_refuse_other_sizes(ops):
     lib = ops.library.load()
-    assert lib.qil_gemm_bf16_mid_splits(257, 4096, 4096) == 0                    # rows
+    assert lib.qil_gemm_bf16_mid_splits(1025, 4096, 4096) == 0                   # rows
+    # beyond 256 rows the op sends it only the products that the library is slow at
+    assert lib.qil_gemm_bf16_mid_rows_takes(512, 4096, 12288) and lib.qil_gemm_bf16_mid_rows_takes(300, 6144, 4096)
+    assert not lib.qil_gemm_bf16_mid_rows_takes(300, 24576, 4096) and not lib.qil_gemm_bf16_mid_rows_takes(256, 4096, 4096)
+    assert not lib.qil_gemm_bf16_mid_rows_takes(512, 6144, 4096) and not lib.qil_gemm_bf16_mid_rows_takes(513, 1024, 3072)
+    assert not lib.qil_gemm_bf16_mid_rows_takes(300, 4100, 4096)
     assert lib.qil_gemm_bf16_mid_splits(128, 4100, 4096) == 0                    # columns in whole waves
     assert lib.qil_gemm_bf16_mid_splits(128, 4096, 4000) == 0                    # K in whole stages
     assert lib.qil_gemm_bf16_mid_splits(128, 4096, 192) == 0                     # four stages at least
