@@ -8,6 +8,7 @@ every request decoding at a 2,048-token history.  Prints ONE JSON line.
 """
 import argparse
 import json
+import random
 import statistics
 import sys
 import time
@@ -165,6 +166,21 @@ def main():
                     assert all(len(r['token_ids']) == 32 for r in results)
                 engine.close()
                 table[f'{length}x{count}'] = round(32 * count / statistics.median(times[1:]), 1)
+        # A mixed batch: 8 requests with prompts of 16 to 2,048 tokens (seeded), portions of 128 under a budget of 512
+        # tokens, 8 active, 32 output tokens each.
+        lengths = [random.Random(7 + i).randrange(16, 2049) for i in range(8)]
+        engine = Engine(model, num_pages=sum(-(-(n + 32) // 16) for n in lengths) + 8, page_size=16, token_budget=512,
+                        prefill_chunk=128, max_active=8)
+        times = []
+        for attempt in range(4):
+            prompts = [prompt(n) for n in lengths]
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            results = engine.generate(prompts, max_new_tokens=32, ignore_eos=True)
+            times.append(time.perf_counter() - started)
+            assert all(len(r['token_ids']) == 32 for r in results)
+        engine.close()
+        table['16-2048x8'] = round(32 * 8 / statistics.median(times[1:]), 1)
         print(json.dumps({'e2e_output_tokens_per_s': table, 'sizes': NAMES[args.sizes], 'layers': args.layers,
                           'dtype': args.dtype}))
         return 0
